@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define MI355_ABI_VERSION 4
+#define MI355_ABI_VERSION 5
 
 typedef void* mi355_stream_t; /* hipStream_t */
 

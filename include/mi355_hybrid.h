@@ -15,7 +15,8 @@ extern "C" {
  * libmi355_hybrid.so: dense linears on [out, in] weights and the kernels of the hybrid decoder family (parallel-residual layers
  * over an fp32 stream; token mixers: paged chunk-masked attention with a softmax sink and position-rotated values, and gated
  * linear recurrences with fp32 state slots; low-rank latent attention over one cached row per token, fixed-decay retention, PolyNorm,
- * sigmoid-gated branches, group-limited mixtures of experts over grouped linears).  act_dtype is MI355_ACT_BF16 or MI355_ACT_F32.  Sources: csrc/gemm_dense.hip,
+ * sigmoid-gated branches, group-limited mixtures of experts over grouped linears; sliding-window and score-capped attention with per-head output gates,
+ * normed queries and keys, a generalized delta-rule recurrence, hashed bigram embedding rows, a weighted average over the depth of the stack).  act_dtype is MI355_ACT_BF16 or MI355_ACT_F32.  Sources: csrc/gemm_dense.hip,
  * csrc/hybrid_ops.hip; the argument conventions are documented at the definitions. */
 int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y, int32_t ldy,
                        int32_t out_f32, int32_t gated, int32_t act, float softcap, int32_t act_dtype, mi355_stream_t stream);
@@ -59,6 +60,31 @@ int mi355_hy_moe_route_align(const float* z, int32_t ld, int32_t tokens, int32_t
                              int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles, mi355_stream_t stream);
 int mi355_hy_moe_combine(const float* y, int32_t tokens, int32_t W, const int32_t* place_of, const float* wts, int32_t top, const float* extra, float* out,
                          mi355_stream_t stream);
+
+/* Extended forms (optional steps as arguments; the short forms above call them with the steps switched off). */
+int mi355_hy_embed_bigram(const int32_t* ids, int32_t rows, const void* table, int32_t W, int32_t vocab, float* out, const int32_t* prev,
+                          const void* bigram, int32_t buckets, int64_t mul_prev, int64_t mul_cur, float* out2, int32_t act_dtype,
+                          mi355_stream_t stream);
+int mi355_hy_depth_mix_norm(float* x, const float* a, float* stack, int64_t plane, int32_t n, const float* coef, const int32_t* rows,
+                            int32_t rows_n, int32_t W, const void* w1, float weight_offset, float eps, void* h1, int32_t act_dtype,
+                            mi355_stream_t stream);
+int mi355_hy_attn_prep_ex(float* qkv, int32_t ld, int32_t koff, int32_t voff, const int32_t* geom, const float* kfreq, const float* vfreq,
+                          int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
+                          void* kcache, void* vcache, const void* qnorm, const void* knorm, float mag, float qt_coef, int32_t qt_every,
+                          int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_attn_rows_ex(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
+                          const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
+                          const void* vcache, void* out, int32_t splits, float* parts, int32_t window, float softcap, const float* ogate,
+                          int32_t ldg, int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_attn_tiles_ex(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
+                           const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0, const int32_t* tile_n,
+                           int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t window, float softcap, const float* ogate,
+                           int32_t ldg, int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_head_norm_ex(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
+                          int32_t goff, void* out, int32_t w_heads, int32_t gate_sigmoid, int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_delta_scan(const float* proj, int32_t ld, int32_t ro, int32_t ko, int32_t vo, int32_t ao, const float* z, int32_t ldz,
+                        float decay_mult, float unit_eps, int32_t H, int32_t dim, int32_t vdim, const int32_t* row_start, const int32_t* slot,
+                        const int32_t* first_pos, int32_t nseq, float* state, float* out, mi355_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -19,7 +19,7 @@ ACT_F16, ACT_BF16, ACT_F32 = 0, 1, 2
 EPI_NONE, EPI_SILU_MUL, EPI_OUT_F32, EPI_OUT_IMAGE = 0, 1, 2, 4
 PF_QKV, PF_O, PF_GATE_UP, PF_QKV_LATE, PF_O_LATE, PF_TP_COMM, PF_TP_INLAUNCH, PF_QKV_IN_FOLD = 1, 2, 4, 16, 32, 64, 128, 256   # mi355_decoder_set_weight_prefetch mask bits
 HINT_STAGED, HINT_NO_PERSISTENT = 0x100, 0x200
-ABI_VERSION = 4
+ABI_VERSION = 5
 KC_NAMES = ["gemm_quant", "gemm_lmhead", "attn", "rope_kv", "norm", "other", "comm"]
 
 vp, i32, f32, sz = C.c_void_p, C.c_int32, C.c_float, C.c_size_t
@@ -182,6 +182,13 @@ HYBRID_SIGNATURES = {
     "mi355_hy_moe_align": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, vp]),
     "mi355_hy_moe_route_align": (i32, [vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp]),
     "mi355_hy_moe_combine": (i32, [vp, i32, i32, vp, vp, i32, vp, vp, vp]),
+    "mi355_hy_embed_bigram": (i32, [vp, i32, vp, i32, i32, vp, vp, vp, i32, C.c_int64, C.c_int64, vp, i32, vp]),
+    "mi355_hy_depth_mix_norm": (i32, [vp, vp, vp, C.c_int64, i32, vp, vp, i32, i32, vp, f32, f32, vp, i32, vp]),
+    "mi355_hy_attn_prep_ex": (i32, [vp, i32, i32, i32, ip, vp, vp, i32, f32, vp, vp, vp, i32, vp, vp, vp, vp, f32, f32, i32, i32, vp]),
+    "mi355_hy_attn_rows_ex": (i32, [vp, i32, f32, ip, i32, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, i32, f32, vp, i32, i32, vp]),
+    "mi355_hy_attn_tiles_ex": (i32, [vp, i32, f32, ip, i32, vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, f32, vp, i32, i32, vp]),
+    "mi355_hy_head_norm_ex": (i32, [vp, i32, i32, i32, vp, f32, vp, i32, i32, vp, i32, i32, i32, vp]),
+    "mi355_hy_delta_scan": (i32, [vp, i32, i32, i32, i32, i32, vp, i32, f32, f32, i32, i32, i32, vp, vp, vp, i32, vp, vp, vp]),
 }
 
 _lib = None

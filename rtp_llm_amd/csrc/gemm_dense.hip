@@ -17,7 +17,7 @@
 
 namespace {
 
-constexpr int DN_ACT_NONE = 0, DN_ACT_RELU = 1, DN_ACT_SILU = 2;
+constexpr int DN_ACT_NONE = 0, DN_ACT_RELU = 1, DN_ACT_SILU = 2, DN_ACT_GELU_TANH = 3, DN_ACT_TANH = 4;
 
 struct DenseParams {
     const void* x; const void* w; const void* bias; void* y;
@@ -57,6 +57,8 @@ __device__ __forceinline__ DnGroup dn_group(const DenseParams& p, int tile_rows)
 __device__ __forceinline__ float dn_act(float g, int act) {
     if (act == DN_ACT_RELU) return g > 0.f ? g : 0.f;
     if (act == DN_ACT_SILU) return g / (1.f + __expf(-g));
+    if (act == DN_ACT_GELU_TANH) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    if (act == DN_ACT_TANH) return tanhf(g);
     return g;
 }
 
@@ -464,15 +466,15 @@ __global__ __launch_bounds__(512) void dense_skinny_bf16_kernel(DenseParams p, i
 
 // x [M, K] (row stride ldx) and w [N, K] of act_dtype (MI355_ACT_BF16 or MI355_ACT_F32); bias [N] of act_dtype or null;
 // y [M, N or N / 2] fp32 (out_f32) or act_dtype, row stride ldy.  gated: the N weight rows are groups of 64 = 32 gate rows followed by
-// the 32 up rows of the same channels (N % 64 == 0); y[m, c] = act(gate_c) * up_c.  act: 0 none, 1 relu, 2 silu (on the gate, or on
-// the plain output).  softcap > 0: y <- softcap * tanh(y / softcap).
+// the 32 up rows of the same channels (N % 64 == 0); y[m, c] = act(gate_c) * up_c.  act: 0 none, 1 relu, 2 silu, 3 gelu (tanh form), 4 tanh (on the gate,
+// or on the plain output).  softcap > 0: y <- softcap * tanh(y / softcap).
 extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias,
                                   void* y, int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, float softcap,
                                   int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(x && w && y && M > 0 && N > 0 && K > 0 && ldx >= K, "dense_linear: M=%d N=%d K=%d ldx=%d", M, N, K, ldx);
     MI355_CHECK_ARG(act_dtype == MI355_ACT_BF16 || act_dtype == MI355_ACT_F32, "dense_linear: act_dtype=%d (bf16 or fp32)", act_dtype);
     MI355_CHECK_ARG(!gated || N % 64 == 0, "dense_linear: gated needs N %% 64 == 0 (N=%d)", N);
-    MI355_CHECK_ARG(act >= 0 && act <= 2, "dense_linear: act=%d", act);
+    MI355_CHECK_ARG(act >= 0 && act <= 4, "dense_linear: act=%d", act);
     MI355_CHECK_ARG(ldy >= (gated ? N / 2 : N), "dense_linear: ldy=%d", ldy);
     const bool bf = act_dtype == MI355_ACT_BF16;
     const size_t es = bf ? 2 : 4;
@@ -524,7 +526,7 @@ extern "C" int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const 
     MI355_CHECK_ARG(ldx >= xs * (G - 1) + K, "dense_grouped: ldx=%d for %d groups of K=%d at step %lld", ldx, G, K, (long long)xs);
     MI355_CHECK_ARG(act_dtype == MI355_ACT_BF16 || act_dtype == MI355_ACT_F32, "dense_grouped: act_dtype=%d (bf16 or fp32)", act_dtype);
     MI355_CHECK_ARG(!gated || N % 64 == 0, "dense_grouped: gated needs N %% 64 == 0 (N=%d)", N);
-    MI355_CHECK_ARG(act >= 0 && act <= 2, "dense_grouped: act=%d", act);
+    MI355_CHECK_ARG(act >= 0 && act <= 4, "dense_grouped: act=%d", act);
     MI355_CHECK_ARG(ldy >= ys * (G - 1) + (gated ? N / 2 : N), "dense_grouped: ldy=%d", ldy);
     MI355_CHECK_ARG(G <= 65535 && (!gather || offs) && (!tiles || (offs && max_tiles > 0)), "dense_grouped: G=%d, gather and tiles need offs", G);
     const bool bf = act_dtype == MI355_ACT_BF16;

@@ -58,12 +58,25 @@ __device__ __forceinline__ void hy_pair(int layout, int i, int n, int& c0, int& 
 }
 
 // ------------------------------------------------------------------------------------------------ embedding -> fp32 stream
+// bigram non-null: the row also takes the table row ((previous token * mul_prev + token * mul_cur) mod buckets), or row `buckets` for a
+// sequence's first token (prev < 0); the sum is formed in fp32.  out2 non-null: a second copy of the rows.
 template <typename T>
-__global__ __launch_bounds__(256) void hy_embed_kernel(const int32_t* ids, const T* table, int W, int vocab, float* out) {
+__global__ __launch_bounds__(256) void hy_embed_kernel(const int32_t* ids, const T* table, int W, int vocab, float* out, const int32_t* prev, const T* bigram,
+                                                       int buckets, unsigned long long mul_prev, unsigned long long mul_cur, float* out2) {
     const int r = blockIdx.x;
     int id = ids[r];
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-    for (int c = threadIdx.x; c < W; c += 256) out[(size_t)r * W + c] = (float)table[(size_t)id * W + c];
+    size_t br = 0;
+    if (bigram) {
+        const int pv = prev[r];
+        br = pv < 0 ? (size_t)buckets : (size_t)(((unsigned long long)pv * mul_prev + (unsigned long long)id * mul_cur) % (unsigned long long)buckets);
+    }
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float v = (float)table[(size_t)id * W + c];
+        if (bigram) v += (float)bigram[br * W + c];
+        out[(size_t)r * W + c] = v;
+        if (out2) out2[(size_t)r * W + c] = v;
+    }
 }
 
 // ------------------------------------------------------------------------------------------------ residual update + one or two norms
@@ -149,6 +162,55 @@ __global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const f
     }
 }
 
+// ------------------------------------------------------------------------------------------------ residual update + weighted average over depth + norm
+// A layer's own result X_n = x + a (a: the layer's last branch, may be null) joins the per-step stack of earlier results (stack[j] = X_j, planes
+// of `plane` floats; X_0 is the embedding output), and what the next layer reads is x <- sum_{j <= n} coef[j] X_j, summed in the order j = 0 .. n in
+// fp32; then h1 = x / rms(x) * (off + w1).  With `rows` only the listed rows are formed and neither x nor the stack is written (the final norm of
+// the rows whose logits are asked for).
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void hy_depth_mix_norm_kernel(float* x, const float* a, float* stack, size_t plane, int n, const float* coef,
+                                                                const int32_t* rows, const T* w1, float off, float eps, int W, T* h1) {
+    extern __shared__ __attribute__((aligned(16))) float hy_xs[];
+    __shared__ float red[4];
+    const int r = blockIdx.x, src = rows ? rows[r] : r;
+    constexpr int V = VEC ? 4 : 1;
+    float ss = 0.f;
+    for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+        const size_t i = (size_t)src * W + c;
+        float v[4], ya[4] = {0.f, 0.f, 0.f, 0.f}, acc[4] = {0.f, 0.f, 0.f, 0.f};
+        if (VEC) { hy_load4<float>(x + i, v); if (a) hy_load4<float>(a + i, ya); }
+        else     { v[0] = x[i]; if (a) ya[0] = a[i]; }
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = v[e] + ya[e];
+        if (!rows) { if (VEC) hy_store4<float>(stack + (size_t)n * plane + i, v); else stack[(size_t)n * plane + i] = v[0]; }
+        for (int j = 0; j < n; ++j) {
+            const float cj = coef[j];
+            float t[4] = {0.f, 0.f, 0.f, 0.f};
+            if (VEC) hy_load4<float>(stack + (size_t)j * plane + i, t); else t[0] = stack[(size_t)j * plane + i];
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc[e] = __builtin_fmaf(cj, t[e], acc[e]);
+        }
+        const float cn = coef[n];
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[e] = __builtin_fmaf(cn, v[e], acc[e]);
+        if (!rows) { if (VEC) hy_store4<float>(x + i, acc); else x[i] = acc[0]; }
+#pragma unroll
+        for (int e = 0; e < V; ++e) { hy_xs[c + e] = acc[e]; ss = __builtin_fmaf(acc[e], acc[e], ss); }
+    }
+    ss = hy_wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    if (!h1) return;
+    const float inv = 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)W + eps);
+    for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+        float g1[4], o1[4];
+        if (VEC) hy_load4<T>(w1 + c, g1); else g1[0] = (float)w1[c];
+#pragma unroll
+        for (int e = 0; e < V; ++e) o1[e] = hy_xs[c + e] * inv * (off + g1[e]);
+        if (VEC) hy_store4<T>(h1 + (size_t)r * W + c, o1); else h1[(size_t)r * W + c] = (T)o1[0];
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ attention: rotate q in place, write K / V pages
 struct AttnGeom {
     int H, G, dim, vdim;
@@ -158,14 +220,31 @@ struct AttnGeom {
     int v_ld;                     // row stride of the value cache in elements (vdim, or wider when the value rows are a part of wider rows)
 };
 
+// Optional steps around the rotation (AttnPrepExtra): a per-head RMS norm of queries and keys under weights shared by the heads (before the
+// rotation), a magnitude on cos and sin, and a position-dependent temperature on the queries, q *= 1 + coef ln(floor((p + 1) / every) + 1).
+struct AttnPrepExtra { const void* qnorm; const void* knorm; float mag; float qt_coef; int qt_every; };
+
 template <typename T>
 __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, int koff, int voff, AttnGeom g, const float* kfreq, const float* vfreq,
                                                            int v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table,
-                                                           T* kcache, T* vcache) {
+                                                           T* kcache, T* vcache, AttnPrepExtra ex) {
     const int r = blockIdx.x, tid = threadIdx.x;
     const int p = pos[r];
     float* row = qkv + (size_t)r * ld;
     const bool has_kv = kcache != nullptr;
+    if (ex.qnorm || (ex.knorm && has_kv)) {           // one wave per head: unit RMS over the head's channels, times the shared weight
+        const int nqh = ex.qnorm ? g.H : 0, nkh = (ex.knorm && has_kv) ? g.G : 0;
+        for (int j = tid >> 6; j < nqh + nkh; j += 4) {
+            const bool isq = j < nqh;
+            float* hd = row + (isq ? j * g.dim : koff + (j - nqh) * g.dim);
+            const T* wn = (const T*)(isq ? ex.qnorm : ex.knorm);
+            float ss = 0.f;
+            for (int c = tid & 63; c < g.dim; c += 64) ss = __builtin_fmaf(hd[c], hd[c], ss);
+            const float inv = 1.f / sqrtf(hy_wave_sum(ss) / (float)g.dim + eps);
+            for (int c = tid & 63; c < g.dim; c += 64) hd[c] = hd[c] * inv * (float)wn[c];
+        }
+        __syncthreads();
+    }
     size_t slot = 0;
     bool slot_ok = false;
     if (has_kv && p >= 0 && p / g.page < g.max_blocks) {
@@ -182,6 +261,7 @@ __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, i
         hy_pair(g.rot_layout, pr, g.rot_dims, c0, c1);
         float sn, cs;
         sincosf(fp * kfreq[pr], &sn, &cs);
+        sn *= ex.mag; cs *= ex.mag;
         float* base = row + (isq ? 0 : koff) + head * g.dim;
         const float u = base[c0], v = base[c1];
         const float ru = u * cs - v * sn, rv = v * cs + u * sn;
@@ -190,6 +270,11 @@ __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, i
             T* kd = kcache + (slot + (size_t)head * g.page) * g.dim;
             kd[c0] = (T)ru; kd[c1] = (T)rv;
         }
+    }
+    if (ex.qt_coef != 0.f) {                           // the temperature follows the rotation: every channel of every query head
+        __syncthreads();
+        const float temp = 1.f + ex.qt_coef * logf((float)((p + 1) / ex.qt_every) + 1.f);
+        for (int i = tid; i < g.H * g.dim; i += 256) row[i] *= temp;
     }
     if (!has_kv || !slot_ok) return;
     const int pass = g.dim - g.rot_dims;                             // key channels beyond the rotary span
@@ -231,10 +316,18 @@ constexpr int HY_MAX_DIM = 512, HY_MAX_VDIM = 512;
 // lane broadcast, and groups of lanes accumulate the value channels of whole value rows in the same way.
 __device__ __forceinline__ float hy_lane_f(float v, int j) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), j)); }
 
+// Optional parts of the mask, the scores and the output (AttnExtra): window > 0: a row at position i sees keys j with 0 <= i - j < window;
+// softcap > 0: score <- softcap tanh(score / softcap) after the scale; ogate non-null: head h of row r is multiplied by
+// sigmoid(ogate[r * ldg + h]) (fp32 pre-activations, one number per head).
+struct AttnExtra { int window; float softcap; const float* ogate; int ldg; };
+__device__ __forceinline__ int hy_first_visible(int p, int chunk, int window) {
+    return chunk > 0 ? (p / chunk) * chunk : (window > 0 ? max(0, p - window + 1) : 0);
+}
+
 template <typename T>
 __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, const float* sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
-                                                           const T* kcache, const T* vcache, T* out, float* parts) {
+                                                           const T* kcache, const T* vcache, T* out, float* parts, AttnExtra ex) {
     constexpr int NV = HY_MAX_VDIM / 64;
     __shared__ __attribute__((aligned(16))) float q_s[HY_MAX_DIM];
     __shared__ float m_s[16], l_s[16];
@@ -246,7 +339,7 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
     const int32_t* bt = block_table + (size_t)seq[r] * g.max_blocks;
     for (int d = tid; d < g.dim; d += NT) q_s[d] = q[(size_t)r * ldq + h * g.dim + d];
     __syncthreads();
-    const int lo = chunk > 0 ? (p / chunk) * chunk : 0;
+    const int lo = hy_first_visible(p, chunk, ex.window);
     // the sink is a key of (unscaled) score sink[h] that carries no value: wave 0 starts from m = sink[h], l = 1
     float m = (sink && wave == 0 && sp == 0) ? sink[h] : -INFINITY, l = (sink && wave == 0 && sp == 0) ? 1.f : 0.f;
     float acc[NV], facc[8];
@@ -300,11 +393,13 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
                 }
             }
             if (valid) s = sc * scale;
+            if (valid && ex.softcap > 0.f) s = ex.softcap * tanhf(s / ex.softcap);
         } else if (valid) {
             const T* kp = kcache + (size_t)rowi * g.dim;
             float d0 = 0.f;
             for (int d = 0; d < g.dim; ++d) d0 = __builtin_fmaf(q_s[d], (float)kp[d], d0);
             s = d0 * scale;
+            if (ex.softcap > 0.f) s = ex.softcap * tanhf(s / ex.softcap);
         }
         const float mn = fmaxf(m, hy_wave_max(s));
         const float pj = valid ? expf(s - mn) : 0.f;
@@ -376,7 +471,8 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
     for (int w = 1; w < NW; ++w) mm = fmaxf(mm, m_s[w]);
     float lt = 0.f;
     for (int w = 0; w < NW; ++w) lt = __builtin_fmaf(l_s[w], (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm), lt);
-    const float invl = S > 1 ? 1.f : (lt > 0.f ? 1.f / lt : 0.f);
+    float invl = S > 1 ? 1.f : (lt > 0.f ? 1.f / lt : 0.f);
+    if (S == 1 && ex.ogate) invl *= hy_sigmoid(ex.ogate[(size_t)r * ex.ldg + h]);
     for (int c = tid; c < g.vdim; c += NT) {
         float a = 0.f;
         for (int w = 0; w < NW; ++w) a = __builtin_fmaf(acc_s[w][c], (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm), a);
@@ -407,7 +503,7 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
 
 // The S partials of a (row, head) -> the head's output: common maximum, summed denominators, value sums rescaled, then the turn back.
 template <typename T>
-__global__ __launch_bounds__(256) void hy_attn_merge_kernel(const float* parts, int S, AttnGeom g, const float* vfreq, const int32_t* pos, T* out) {
+__global__ __launch_bounds__(256) void hy_attn_merge_kernel(const float* parts, int S, AttnGeom g, const float* vfreq, const int32_t* pos, T* out, AttnExtra ex) {
     __shared__ float o_s[HY_MAX_VDIM];
     const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const float* pd = parts + ((size_t)r * g.H + h) * S * (g.vdim + 2);
@@ -418,7 +514,8 @@ __global__ __launch_bounds__(256) void hy_attn_merge_kernel(const float* parts, 
         const float ms = pd[(size_t)s_ * (g.vdim + 2)];
         lt = __builtin_fmaf(pd[(size_t)s_ * (g.vdim + 2) + 1], (ms == -INFINITY) ? 0.f : expf(ms - mm), lt);
     }
-    const float invl = lt > 0.f ? 1.f / lt : 0.f;
+    float invl = lt > 0.f ? 1.f / lt : 0.f;
+    if (ex.ogate) invl *= hy_sigmoid(ex.ogate[(size_t)r * ex.ldg + h]);
     for (int c = tid; c < g.vdim; c += 256) {
         float a = 0.f;
         for (int s_ = 0; s_ < S; ++s_) {
@@ -474,7 +571,7 @@ template <int DKM, int NCBM, int NWV>     // most 32-channel steps of a key row 
 __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, const float* sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
                                                            const int32_t* tile_row0, const int32_t* tile_n, int ntiles, const bf16* kcache, const bf16* vcache,
-                                                           bf16* out) {
+                                                           bf16* out, AttnExtra ex) {
     __shared__ __attribute__((aligned(16))) bf16 Ph_all[4][16 * AT_LD];
     __shared__ __attribute__((aligned(16))) bf16 Pl_all[4][16 * AT_LD];
     __shared__ __attribute__((aligned(16))) bf16 Vt[NCBM * 16 * AT_LD];
@@ -499,7 +596,9 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
         return (size_t)(bt[pi] * g.G + kvh) * g.page + po;
     };
     // scores are kept times log2(e): the weights are then 2^(s - m), one v_exp_f32 each; the sink (score 0) and the ratios are unchanged
-    const float scale2 = scale * 1.44269504088896340736f;
+    // (with a cap the products come out in natural units, are capped, and only then go to the log2 scale)
+    const float scale2 = ex.softcap > 0.f ? scale : scale * 1.44269504088896340736f;
+    const float cap2 = ex.softcap * 1.44269504088896340736f, icap2 = ex.softcap > 0.f ? 2.f * 1.44269504088896340736f / ex.softcap : 0.f;
     bf16x8 qh[DKM], ql[DKM];
 #pragma unroll
     for (int ks = 0; ks < DKM; ++ks) {
@@ -515,11 +614,11 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
 #pragma unroll
     for (int cb = 0; cb < NCBM; ++cb) o[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int plast = p0 + n - 1;
-    const int rlo_last = chunk > 0 ? (plast / chunk) * chunk : 0;
+    const int rlo_last = hy_first_visible(plast, chunk, ex.window);
     int rlo4[4];                                              // first visible position of the lane's four rows
 #pragma unroll
-    for (int e = 0; e < 4; ++e) rlo4[e] = chunk > 0 ? ((p0 + lq * 4 + e) / chunk) * chunk : 0;
-    const int kstart = (chunk > 0 ? (p0 / chunk) * chunk : 0) & ~31;
+    for (int e = 0; e < 4; ++e) rlo4[e] = hy_first_visible(p0 + lq * 4 + e, chunk, ex.window);
+    const int kstart = hy_first_visible(p0, chunk, ex.window) & ~31;
     // the key fragments and raw value rows of the next 32 keys are fetched while the current 32 are worked on
     bf16x8 kn[2][DKM];
     u32x4 vn[VEM];
@@ -552,6 +651,13 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qh[ks], kn[kb][ks], acc, 0, 0, 0);
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ql[ks], kn[kb][ks], acc, 0, 0, 0);
                 }
+            if (ex.softcap > 0.f) {       // cap tanh(s / cap) = cap (t - 1) / (t + 1), t = 2^(2 s log2(e) / cap), the exponent kept inside fp32's range
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float t = __builtin_amdgcn_exp2f(fminf(fmaxf(acc[e] * icap2, -60.f), 60.f));
+                    acc[e] = cap2 * ((t - 1.f) / (t + 1.f));
+                }
+            }
             s[kb] = acc;
         }
         // the 32 value rows, transposed: Vt[channel][key]; neighbouring lanes write neighbouring keys of one channel row
@@ -614,7 +720,8 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
     for (int e = 0; e < 4; ++e) {
         const int row = lq * 4 + e;
         const float lt = hy_sum16(l[e]);
-        const float inv = lt > 0.f ? 1.f / lt : 0.f;
+        float inv = lt > 0.f ? 1.f / lt : 0.f;
+        if (ex.ogate && row < n) inv *= hy_sigmoid(ex.ogate[(size_t)(r0 + row) * ex.ldg + h]);
         const float fp = (float)(p0 + row);
         bf16* od = out + ((size_t)(r0 + row) * g.H + h) * g.vdim;
 #pragma unroll
@@ -778,9 +885,131 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
     }
 }
 
-// per-head RMS norm over vdim with a plain weight shared by the heads (null: none), optional silu gate: one wave per (row, head)
+// ------------------------------------------------------------------------------------------------ generalized delta rule
+// S_t = diag(w_t) S_(t-1) - (a_t * u_t)(u_t^T S_(t-1)) + k_t v_t^T, o_t = S_t^T r_t per head, S [dim (key channel), vdim] in an fp32 slot; both the
+// decayed and the removed term read the old state.  w = exp(-decay_mult * sigmoid(z)), a = sigmoid(removal pre-activation), u = k / sqrt(|k|^2 +
+// unit_eps) over the head's key channels: all in fp32.  A quad of lanes owns one value column, each lane RD of its key rows; a wave owns 16 columns
+// and a block of four waves 64.  Per token the only exchange is the quad sum of u^T S (and of the output), two DPP steps each; the gates of `tok`
+// tokens are computed once into LDS by the whole block.  The walk over a sequence's tokens is the same arithmetic however the tokens were cut into steps.
+struct DeltaParams {
+    const float* proj; int ld; int ro, ko, vo, ao;   // fp32 projections [rows, ld]: r, k, v heads and the removal pre-activation at these columns
+    const float* z; int ldz;                          // decay pre-activation [rows, H * dim]
+    float decay_mult, unit_eps;
+    int H, dim, vdim;
+    const int32_t* row_start; const int32_t* slot; const int32_t* first_pos;
+    float* state;                                     // [slots, H, dim, vdim]
+    float* out;                                       // [rows, H * vdim]
+    int tok;
+};
+
+__device__ __forceinline__ float hy_quad_sum(float v) {
+    v += hy_dpp<0xB1>(v);      // quad_perm [1,0,3,2]
+    return v + hy_dpp<0x4E>(v);  // quad_perm [2,3,0,1]
+}
+
+template <int RD>
+__global__ __launch_bounds__(256) void hy_delta_kernel(DeltaParams p) {
+    extern __shared__ __attribute__((aligned(16))) float hy_dl[];
+    constexpr int dpad = 4 * RD;
+    const int TOK = p.tok;
+    float* w_s = hy_dl;                          // [TOK][dpad] each
+    float* b_s = w_s + TOK * dpad;
+    float* u_s = b_s + TOK * dpad;
+    float* k_s = u_s + TOK * dpad;
+    float* r_s = k_s + TOK * dpad;
+    float* v_s = r_s + TOK * dpad;               // [TOK][64]
+    float* o_s = v_s + TOK * 64;                 // [TOK][64]
+    float* inv_s = o_s + TOK * 64;               // [TOK]
+    const int sq = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rg = lane & 3, col = wave * 16 + (lane >> 2);
+    const int r0 = p.row_start[sq], r1 = p.row_start[sq + 1];
+    const bool vok = v0 + col < p.vdim;
+    float* st = p.state + (((size_t)p.slot[sq] * p.H + h) * p.dim) * p.vdim + v0 + col;
+    const bool fresh = p.first_pos[sq] == 0;
+    float S[RD];
+#pragma unroll
+    for (int j = 0; j < RD; ++j) {
+        const int d = rg * RD + j;
+        S[j] = (!fresh && vok && d < p.dim) ? st[(size_t)d * p.vdim] : 0.f;
+    }
+    for (int t0 = r0; t0 < r1; t0 += TOK) {
+        const int nt = min(TOK, r1 - t0);
+        for (int i = tid; i < nt * dpad; i += 256) {
+            const int t = i / dpad, d = i % dpad;
+            float rv = 0.f, kv = 0.f, wv = 1.f, av = 0.f;
+            if (d < p.dim) {
+                const float* row = p.proj + (size_t)(t0 + t) * p.ld;
+                const int hd = h * p.dim + d;
+                rv = row[p.ro + hd]; kv = row[p.ko + hd];
+                av = hy_sigmoid(row[p.ao + hd]);
+                wv = expf(-p.decay_mult * hy_sigmoid(p.z[(size_t)(t0 + t) * p.ldz + hd]));
+            }
+            r_s[i] = rv; k_s[i] = kv; w_s[i] = wv; b_s[i] = av;
+        }
+        for (int i = tid; i < nt * 64; i += 256)
+            v_s[i] = (v0 + (i & 63) < p.vdim) ? p.proj[(size_t)(t0 + (i >> 6)) * p.ld + p.vo + h * p.vdim + v0 + (i & 63)] : 0.f;
+        __syncthreads();
+        for (int t = wave; t < nt; t += 4) {         // |k|^2 of a token's head: one wave
+            float ss = 0.f;
+            for (int d = lane; d < p.dim; d += 64) ss = __builtin_fmaf(k_s[t * dpad + d], k_s[t * dpad + d], ss);
+            ss = hy_wave_sum(ss);
+            if (lane == 0) inv_s[t] = 1.f / sqrtf(ss + p.unit_eps);
+        }
+        __syncthreads();
+        for (int i = tid; i < nt * dpad; i += 256) {
+            const float u = k_s[i] * inv_s[i / dpad];
+            u_s[i] = u; b_s[i] = b_s[i] * u;
+        }
+        __syncthreads();
+        for (int t = 0; t < nt; ++t) {
+            const float vt = v_s[t * 64 + col];
+            const f32x4* uu = (const f32x4*)(u_s + t * dpad + rg * RD);
+            const f32x4* ww = (const f32x4*)(w_s + t * dpad + rg * RD);
+            const f32x4* bb = (const f32x4*)(b_s + t * dpad + rg * RD);
+            const f32x4* kk = (const f32x4*)(k_s + t * dpad + rg * RD);
+            const f32x4* rr = (const f32x4*)(r_s + t * dpad + rg * RD);
+            float sp[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j4 = 0; j4 < RD / 4; ++j4) {
+                const f32x4 u4 = uu[j4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sp[e] = __builtin_fmaf(u4[e], S[j4 * 4 + e], sp[e]);
+            }
+            const float sb = hy_quad_sum((sp[0] + sp[1]) + (sp[2] + sp[3]));      // (u^T S_old)[column]
+            float op[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j4 = 0; j4 < RD / 4; ++j4) {
+                const f32x4 w4 = ww[j4], b4 = bb[j4], k4 = kk[j4], r4 = rr[j4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = j4 * 4 + e;
+                    S[j] = __builtin_fmaf(w4[e], S[j], __builtin_fmaf(-b4[e], sb, k4[e] * vt));
+                    op[e] = __builtin_fmaf(r4[e], S[j], op[e]);
+                }
+            }
+            const float o = hy_quad_sum((op[0] + op[1]) + (op[2] + op[3]));
+            if (rg == 0) o_s[t * 64 + col] = o;
+        }
+        __syncthreads();
+        for (int i = tid; i < nt * 64; i += 256) {
+            const int cc = i & 63;
+            if (v0 + cc < p.vdim) p.out[(size_t)(t0 + (i >> 6)) * p.H * p.vdim + h * p.vdim + v0 + cc] = o_s[i];
+        }
+    }
+    if (vok) {
+#pragma unroll
+        for (int j = 0; j < RD; ++j) {
+            const int d = rg * RD + j;
+            if (d < p.dim) st[(size_t)d * p.vdim] = S[j];
+        }
+    }
+}
+
+// per-head RMS norm over vdim with a plain weight (null: none; shared by the heads, or w_heads: one per head and channel, [H * vdim]), optional
+// gate (silu, or gate_sigmoid: sigmoid): one wave per (row, head)
 template <typename T>
-__global__ __launch_bounds__(64) void hy_head_norm_kernel(const float* o, int H, int vdim, const T* w, float eps, const float* gate, int ldg, int goff, T* out) {
+__global__ __launch_bounds__(64) void hy_head_norm_kernel(const float* o, int H, int vdim, const T* w, float eps, const float* gate, int ldg, int goff, T* out,
+                                                          int w_heads, int gate_sigmoid) {
     const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const float* src = o + ((size_t)r * H + h) * vdim;
     float ss = 0.f;
@@ -788,8 +1017,8 @@ __global__ __launch_bounds__(64) void hy_head_norm_kernel(const float* o, int H,
     const float inv = 1.f / sqrtf(hy_wave_sum(ss) / (float)vdim + eps);
     for (int c = lane; c < vdim; c += 64) {
         float v = src[c] * inv;
-        if (w) v *= (float)w[c];
-        if (gate) v *= hy_silu(gate[(size_t)r * ldg + goff + h * vdim + c]);
+        if (w) v *= (float)w[w_heads ? h * vdim + c : c];
+        if (gate) { const float gz = gate[(size_t)r * ldg + goff + h * vdim + c]; v *= gate_sigmoid ? hy_sigmoid(gz) : hy_silu(gz); }
         out[((size_t)r * H + h) * vdim + c] = (T)v;
     }
 }
@@ -1072,8 +1301,19 @@ int hy_geom_ok(const AttnGeom& g) {
 
 extern "C" int mi355_hy_embed(const int32_t* ids, int32_t rows, const void* table, int32_t W, int32_t vocab, float* out, int32_t act_dtype,
                               mi355_stream_t stream) {
+    return mi355_hy_embed_bigram(ids, rows, table, W, vocab, out, nullptr, nullptr, 0, 0, 0, nullptr, act_dtype, stream);
+}
+
+// out[r] = table[ids[r]] (+ bigram[row(prev[r], ids[r])]): fp32 [rows, W]; bigram [buckets + 1, W] of act_dtype with prev int32 [rows] (the token
+// before each row in its sequence, < 0 for a first token: row `buckets`), row = (prev * mul_prev + id * mul_cur) mod buckets in 64-bit arithmetic.
+// out2: null, or a second fp32 [rows, W] that receives the same rows.
+extern "C" int mi355_hy_embed_bigram(const int32_t* ids, int32_t rows, const void* table, int32_t W, int32_t vocab, float* out, const int32_t* prev,
+                                     const void* bigram, int32_t buckets, int64_t mul_prev, int64_t mul_cur, float* out2, int32_t act_dtype,
+                                     mi355_stream_t stream) {
     MI355_CHECK_ARG(ids && table && out && rows > 0 && W > 0 && vocab > 0, "hy_embed: rows=%d W=%d", rows, W);
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_embed_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids, (const T*)table, W, vocab, out));
+    MI355_CHECK_ARG(!bigram || (prev && buckets > 0 && mul_prev >= 0 && mul_cur >= 0), "hy_embed: bigram table of %d buckets", buckets);
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_embed_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids, (const T*)table, W, vocab, out, prev,
+                                              (const T*)bigram, buckets, (unsigned long long)mul_prev, (unsigned long long)mul_cur, out2));
     MI355_CHECK_LAUNCH("hy_embed_kernel");
     return MI355_OK;
 }
@@ -1109,19 +1349,51 @@ extern "C" int mi355_hy_residual_norm(float* x, const float* a, const float* b, 
     return mi355_hy_gated_residual_norm(x, a, b, nullptr, 0, mult, rows, n, W, w1, w2, weight_offset, eps, h1, h2, nullptr, nullptr, nullptr, 0, act_dtype, stream);
 }
 
+// x fp32 [T, W] stream (the layer's input plus its earlier branches), a fp32 [T, W] or null; stack fp32 [>= n + 1, T, W] with planes 0 .. n - 1 filled;
+// coef fp32 [n + 1] on the device.  Writes stack[n] = x + a, x = sum_j coef[j] stack[j], h1 [rows_n, W] of act_dtype (null: no norm).  rows: null
+// (rows_n = T rows, in place), or rows_n row indices to form without writing x or the stack.
+extern "C" int mi355_hy_depth_mix_norm(float* x, const float* a, float* stack, int64_t plane, int32_t n, const float* coef, const int32_t* rows,
+                                       int32_t rows_n, int32_t W, const void* w1, float weight_offset, float eps, void* h1, int32_t act_dtype,
+                                       mi355_stream_t stream) {
+    MI355_CHECK_ARG(x && stack && coef && rows_n > 0 && W > 0 && n >= 0 && plane >= W && (!h1 || w1), "hy_depth_mix_norm: rows=%d W=%d n=%d", rows_n, W, n);
+    MI355_CHECK_ARG((size_t)W * 4 <= 64 * 1024, "hy_depth_mix_norm: W=%d too wide for one block", W);
+    auto al = [](const void* p_) { return ((uintptr_t)p_ & 15) == 0; };
+    if (W % 4 == 0 && plane % 4 == 0 && al(x) && al(a) && al(stack) && al(w1) && al(h1))
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_depth_mix_norm_kernel<T, true>), dim3(rows_n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, stack,
+                                                  (size_t)plane, n, coef, rows, (const T*)w1, weight_offset, eps, W, (T*)h1));
+    else
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_depth_mix_norm_kernel<T, false>), dim3(rows_n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, stack,
+                                                  (size_t)plane, n, coef, rows, (const T*)w1, weight_offset, eps, W, (T*)h1));
+    MI355_CHECK_LAUNCH("hy_depth_mix_norm_kernel");
+    return MI355_OK;
+}
+
 // geom: {H, G, dim, vdim, rot_dims, rot_layout, v_layout, page, max_blocks, num_pages}.  qkv fp32 [rows, ld]: q heads at column 0 (rotated in
 // place), k heads at koff, v heads at voff.  kcache [pages, G, page, dim], vcache [pages, G, page, vdim] of act_dtype; null kcache: queries only
 // (a layer that reads another layer's cache).  kfreq [rot_dims / 2], vfreq [vdim / 2] fp32 angular steps (vfreq null: values are not rotated).
 extern "C" int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t voff, const int32_t* geom, const float* kfreq, const float* vfreq,
                                   int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
                                   void* kcache, void* vcache, int32_t act_dtype, mi355_stream_t stream) {
+    return mi355_hy_attn_prep_ex(qkv, ld, koff, voff, geom, kfreq, vfreq, v_norm, eps, pos, seq, block_table, rows, kcache, vcache, nullptr, nullptr, 1.f, 0.f, 1,
+                                 act_dtype, stream);
+}
+
+// The same with the optional steps: qnorm / knorm (act_dtype [dim], or null): queries / keys are brought to unit RMS per head (eps) and multiplied
+// by the weight before the rotation; mag multiplies cos and sin; qt_coef != 0: queries are multiplied by 1 + qt_coef ln(floor((p + 1) / qt_every) + 1)
+// after the rotation.
+extern "C" int mi355_hy_attn_prep_ex(float* qkv, int32_t ld, int32_t koff, int32_t voff, const int32_t* geom, const float* kfreq, const float* vfreq,
+                                     int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
+                                     void* kcache, void* vcache, const void* qnorm, const void* knorm, float mag, float qt_coef, int32_t qt_every,
+                                     int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(qkv && geom && pos && seq && rows > 0, "hy_attn_prep: null argument");
+    MI355_CHECK_ARG(qt_coef == 0.f || qt_every > 0, "hy_attn_prep: query temperature every %d positions", qt_every);
+    const AttnPrepExtra ex{qnorm, knorm, mag, qt_coef, qt_every};
     const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
     MI355_CHECK_ARG((g.rot_dims == 0 || kfreq) && (!kcache || (vcache && block_table)), "hy_attn_prep: missing table or cache");
     MI355_CHECK_ARG(!vfreq || g.vdim % 2 == 0, "hy_attn_prep: rotated values need an even value size (%d)", g.vdim);
     HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_prep_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, qkv, ld, koff, voff, g, kfreq, vfreq,
-                                              v_norm, eps, pos, seq, block_table, (T*)kcache, (T*)vcache));
+                                              v_norm, eps, pos, seq, block_table, (T*)kcache, (T*)vcache, ex));
     MI355_CHECK_LAUNCH("hy_attn_prep_kernel");
     return MI355_OK;
 }
@@ -1133,6 +1405,18 @@ extern "C" int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t 
 extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
                                   const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
                                   const void* vcache, void* out, int32_t splits, float* parts, int32_t act_dtype, mi355_stream_t stream) {
+    return mi355_hy_attn_rows_ex(q, ldq, scale, geom, chunk, sink, vfreq, pos, seq, block_table, rows, kcache, vcache, out, splits, parts, 0, 0.f, nullptr, 0,
+                                 act_dtype, stream);
+}
+
+// The same with a sliding window (window > 0, chunk must be 0: keys j with 0 <= i - j < window), a tanh cap on the scaled scores (softcap > 0) and a
+// sigmoid gate per (row, head) on the output (ogate fp32 [rows, ldg], column h; null: none).
+extern "C" int mi355_hy_attn_rows_ex(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
+                                     const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
+                                     const void* vcache, void* out, int32_t splits, float* parts, int32_t window, float softcap, const float* ogate,
+                                     int32_t ldg, int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(window >= 0 && (window == 0 || chunk == 0) && softcap >= 0.f && (!ogate || ldg >= geom[0]), "hy_attn_rows: window=%d chunk=%d ldg=%d", window, chunk, ldg);
+    const AttnExtra ex{window, softcap, ogate, ldg};
     MI355_CHECK_ARG(q && geom && pos && seq && block_table && kcache && vcache && out && rows > 0 && chunk >= 0, "hy_attn_rows: bad argument");
     MI355_CHECK_ARG(splits >= 1 && splits <= 64 && (splits == 1 || parts), "hy_attn_rows: %d splits", splits);
     MI355_CHECK_ARG(!vfreq || geom[3] % 2 == 0, "hy_attn_rows: rotated values need an even value size (%d)", geom[3]);
@@ -1140,10 +1424,10 @@ extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, cons
     if (int e = hy_geom_ok(g)) return e;
     const int threads = rows * g.H <= 2048 ? 1024 : 256;     // few (decode) rows: sixteen waves share a row's keys
     HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H, splits), dim3(threads), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
-                                              pos, seq, block_table, (const T*)kcache, (const T*)vcache, (T*)out, parts));
+                                              pos, seq, block_table, (const T*)kcache, (const T*)vcache, (T*)out, parts, ex));
     MI355_CHECK_LAUNCH("hy_attn_rows_kernel");
     if (splits > 1) {
-        HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_merge_kernel<T>, dim3(rows, g.H), dim3(256), 0, (hipStream_t)stream, parts, splits, g, vfreq, pos, (T*)out));
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_merge_kernel<T>, dim3(rows, g.H), dim3(256), 0, (hipStream_t)stream, parts, splits, g, vfreq, pos, (T*)out, ex));
         MI355_CHECK_LAUNCH("hy_attn_merge_kernel");
     }
     return MI355_OK;
@@ -1155,6 +1439,16 @@ extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, con
                                    const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0,
                                    const int32_t* tile_n, int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t act_dtype,
                                    mi355_stream_t stream) {
+    return mi355_hy_attn_tiles_ex(q, ldq, scale, geom, chunk, sink, vfreq, pos, seq, block_table, tile_row0, tile_n, tiles, kcache, vcache, out, 0, 0.f, nullptr, 0,
+                                  act_dtype, stream);
+}
+
+extern "C" int mi355_hy_attn_tiles_ex(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
+                                      const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0,
+                                      const int32_t* tile_n, int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t window, float softcap,
+                                      const float* ogate, int32_t ldg, int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(window >= 0 && (window == 0 || chunk == 0) && softcap >= 0.f && (!ogate || ldg >= geom[0]), "hy_attn_tiles: window=%d chunk=%d ldg=%d", window, chunk, ldg);
+    const AttnExtra ex{window, softcap, ogate, ldg};
     MI355_CHECK_ARG(q && geom && pos && seq && block_table && tile_row0 && tile_n && kcache && vcache && out && tiles > 0 && chunk >= 0, "hy_attn_tiles: bad argument");
     const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
@@ -1165,7 +1459,7 @@ extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, con
     const int gq = g.H / g.G, nwv = gq % 4 == 0 ? 4 : gq % 2 == 0 ? 2 : 1;       // query heads of one key/value head per block
 #define HY_TILES(DKM_, NCBM_, NWV_)                                                                                                            \
     hipLaunchKernelGGL((hy_attn_tiles_kernel<DKM_, NCBM_, NWV_>), dim3((tiles + 1) / 2, g.H / NWV_), dim3(64 * NWV_), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, \
-                       sink, vfreq, pos, seq, block_table, tile_row0, tile_n, tiles, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out)
+                       sink, vfreq, pos, seq, block_table, tile_row0, tile_n, tiles, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out, ex)
     if (g.dim <= 128 && g.vdim <= 128) { if (nwv == 4) HY_TILES(4, 8, 4); else if (nwv == 2) HY_TILES(4, 8, 2); else HY_TILES(4, 8, 1); }
     else                               { if (nwv == 4) HY_TILES(8, 16, 4); else if (nwv == 2) HY_TILES(8, 16, 2); else HY_TILES(8, 16, 1); }
 #undef HY_TILES
@@ -1201,11 +1495,43 @@ extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_
     return MI355_OK;
 }
 
+// proj fp32 [rows, ld]: receptance r, key k (H heads of dim) at columns ro, ko, value v (H heads of vdim) at vo, removal pre-activation (H heads of dim,
+// bias included) at ao; z fp32 [rows, ldz]: decay pre-activation (H heads of dim, bias included).  w = exp(-decay_mult sigmoid(z)), a = sigmoid(.),
+// u = k / sqrt(|k|^2 + unit_eps).  Sequences, slots and the state [slots, H, dim, vdim] as in mi355_hy_scan.  out fp32 [rows, H * vdim].  dim <= 256.
+extern "C" int mi355_hy_delta_scan(const float* proj, int32_t ld, int32_t ro, int32_t ko, int32_t vo, int32_t ao, const float* z, int32_t ldz,
+                                   float decay_mult, float unit_eps, int32_t H, int32_t dim, int32_t vdim, const int32_t* row_start, const int32_t* slot,
+                                   const int32_t* first_pos, int32_t nseq, float* state, float* out, mi355_stream_t stream) {
+    MI355_CHECK_ARG(proj && z && row_start && slot && first_pos && state && out && nseq > 0 && H > 0 && dim > 0 && vdim > 0, "hy_delta_scan: bad argument");
+    MI355_CHECK_ARG(dim <= 256, "hy_delta_scan: key size %d > 256", dim);
+    MI355_CHECK_ARG(ld >= H * dim && ldz >= H * dim && unit_eps >= 0.f, "hy_delta_scan: ld=%d ldz=%d", ld, ldz);
+    const int RD = dim <= 16 ? 4 : dim <= 32 ? 8 : dim <= 64 ? 16 : dim <= 128 ? 32 : 64;
+    int tok = 16;
+    auto lds_of = [&](int t) { return (size_t)(5 * t * 4 * RD + 2 * t * 64 + t) * 4; };
+    while (tok > 1 && lds_of(tok) > 60 * 1024) tok >>= 1;
+    DeltaParams p{proj, ld, ro, ko, vo, ao, z, ldz, decay_mult, unit_eps, H, dim, vdim, row_start, slot, first_pos, state, out, tok};
+    const dim3 grid(nseq, H, (vdim + 63) / 64);
+    const size_t lds = lds_of(tok);
+    hipStream_t st = (hipStream_t)stream;
+    if (RD == 4)       hipLaunchKernelGGL(hy_delta_kernel<4>, grid, dim3(256), lds, st, p);
+    else if (RD == 8)  hipLaunchKernelGGL(hy_delta_kernel<8>, grid, dim3(256), lds, st, p);
+    else if (RD == 16) hipLaunchKernelGGL(hy_delta_kernel<16>, grid, dim3(256), lds, st, p);
+    else if (RD == 32) hipLaunchKernelGGL(hy_delta_kernel<32>, grid, dim3(256), lds, st, p);
+    else               hipLaunchKernelGGL(hy_delta_kernel<64>, grid, dim3(256), lds, st, p);
+    MI355_CHECK_LAUNCH("hy_delta_kernel");
+    return MI355_OK;
+}
+
 extern "C" int mi355_hy_head_norm(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
                                   int32_t goff, void* out, int32_t act_dtype, mi355_stream_t stream) {
+    return mi355_hy_head_norm_ex(o, rows, H, vdim, w, eps, gate, ldg, goff, out, 0, 0, act_dtype, stream);
+}
+
+// w_heads: w is [H * vdim] (a weight per head and channel) instead of [vdim]; gate_sigmoid: the gate is sigmoid(gate) instead of silu(gate).
+extern "C" int mi355_hy_head_norm_ex(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
+                                     int32_t goff, void* out, int32_t w_heads, int32_t gate_sigmoid, int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(o && out && rows > 0 && H > 0 && vdim > 0, "hy_head_norm: bad argument");
     HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_head_norm_kernel<T>, dim3(rows, H), dim3(64), 0, (hipStream_t)stream, o, H, vdim, (const T*)w, eps, gate, ldg,
-                                              goff, (T*)out));
+                                              goff, (T*)out, w_heads, gate_sigmoid));
     MI355_CHECK_LAUNCH("hy_head_norm_kernel");
     return MI355_OK;
 }

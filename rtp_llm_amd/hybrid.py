@@ -11,7 +11,11 @@ final.norm, head) and runs one ragged step against the cache tensors an engine a
 Members: Nufalorn (chunk-masked sink attention with unit-normed, rotated values and shared-KV layers, HGRN2 and GLA recurrences,
 relu-gated MLPs, two offset norms per layer) and Pokepel (latent attention and retention, PolyNorm MLPs and group-limited mixtures of
 silu-gated experts with a shared expert, one plain norm per layer, sigmoid-gated branches; checkpoint tensors l<i>.rg1 / rg2 (+ .b),
-l<i>.mlp.{up, down, act} or l<i>.mlp.{router, e<j>.{gate, up, down}, shared.{gate, up, down}})."""
+l<i>.mlp.{up, down, act} or l<i>.mlp.{router, e<j>.{gate, up, down}, shared.{gate, up, down}}) and Nepudra (sequential pre-norm layers
+x <- x + mixer(norm1 x), x <- x + mlp(norm2 x) whose norms have ONE gain for all channels, every layer reading a learned weighted average
+of the embedding output and the results of all layers before it (l<i>.dwa); a hashed bigram table beside the token embedding (bigram);
+mixers: a generalized delta-rule recurrence, causal attention with a query temperature, a score cap, biases and per-head output gates, and
+sliding-window attention with normed, YaRN-rotated queries and keys; gelu-gated MLPs)."""
 import json
 import os
 from dataclasses import dataclass, field
@@ -20,19 +24,28 @@ from typing import Dict, List, Optional, Union
 import torch
 
 from . import hybrid_ops as hops
-from .mixers import (AttentionSpec, GatedLinearRecurrence, GatedMLP, LatentAttention, LatentAttentionSpec, PagedChunkAttention, PolyNormMLP,
-                     RecurrenceSpec, Retention, RetentionSpec, RotarySpec, RoutedExperts, RouterSpec, StepBatch)
+from .mixers import (AttentionSpec, DeltaRuleSpec, GatedLinearRecurrence, GatedMLP, GeneralizedDeltaRule, LatentAttention, LatentAttentionSpec,
+                     PagedChunkAttention, PolyNormMLP, RecurrenceSpec, Retention, RetentionSpec, RotarySpec, RoutedExperts, RouterSpec, StepBatch)
 
 
 @dataclass
 class HybridLayerSpec:
-    kind: str                                        # "attention" | "hgrn2" | "gla" | "latent_attention" | "retention"
-    mixer: Union[AttentionSpec, RecurrenceSpec, LatentAttentionSpec, RetentionSpec]
+    kind: str                                        # "attention" | "hgrn2" | "gla" | "latent_attention" | "retention" | "delta_rule"
+    mixer: Union[AttentionSpec, RecurrenceSpec, LatentAttentionSpec, RetentionSpec, DeltaRuleSpec]
     ff: Optional[int] = None                         # None: the layer has no MLP; hidden size of the dense MLP or of one routed expert
     mlp_act: str = "relu"
     mlp_kind: str = "gated"                          # "gated" | "polynorm" | "experts"
     router: Optional[RouterSpec] = None              # experts: the router ...
     shared_ff: Optional[int] = None                  # ... and the hidden size of the expert every token runs (None: no such expert)
+
+
+@dataclass
+class BigramSpec:
+    """A second embedding table indexed by a hash of (previous token, token): row (prev * mul_prev + token * mul_cur) mod buckets, and row
+    `buckets` (the table's last) for the first token of a sequence."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
 
 
 @dataclass
@@ -47,6 +60,10 @@ class HybridConfig:
     norm_offset: float = 1.0                         # stored norm weights are offsets from this value
     shared_norm: bool = False                        # one norm per layer feeds the mixer and the MLP
     branch_gates: bool = False                       # each branch is multiplied by sigmoid(W h + b) of its input before it joins the stream
+    sequential: bool = False                         # x <- x + mixer(norm1 x), then x <- x + mlp(norm2 x) (instead of both branches from one x)
+    scalar_norm: bool = False                        # every norm's weight is ONE number for all channels
+    depth_mix: bool = False                          # a layer reads sum_j dwa[j] X_j over the embedding output X_0 and all earlier layers' results
+    bigram: Optional[BigramSpec] = None              # hashed (previous token, token) rows added to the token embedding
 
     @staticmethod
     def from_json(cfg: dict) -> "HybridConfig":
@@ -78,12 +95,7 @@ class HybridConfig:
             if mlp is not None and mlp.get("kind", "dense") != "dense":
                 raise NotImplementedError(f"layer {i}: mlp kind {mlp.get('kind')!r}")
             layers.append(HybridLayerSpec(kind, spec, None if mlp is None else int(mlp["ff"]), "relu"))
-        for i, L in enumerate(layers):
-            src = getattr(L.mixer, "kv_from", None)
-            if src is not None:
-                o = layers[src].mixer if 0 <= src < i else None
-                if not isinstance(o, AttentionSpec) or o.kv_from is not None or (o.kv_heads, o.dim, o.vdim) != (L.mixer.kv_heads, L.mixer.dim, L.mixer.vdim):
-                    raise ValueError(f"layer {i}: kv_from {src} must name an earlier attention layer with its own keys and values of the same shape")
+        _check_kv_from(layers)
         return HybridConfig(name=str(cfg.get("architecture", "hybrid")), vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=layers,
                             eps=float(cfg["norm"]["eps"]), residual_mult=float(cfg.get("residual_mult", 1.0)),
                             logit_softcap=float(cfg.get("logit_softcap") or 0.0))
@@ -124,7 +136,50 @@ class HybridConfig:
                             residual_mult=1.0, logit_softcap=0.0, norm_offset=0.0, shared_norm=True, branch_gates=True)
 
 
-_READERS = {"nufalorn": HybridConfig.nufalorn_from_json, "pokepel": HybridConfig.pokepel_from_json}
+def _check_kv_from(layers):
+    for i, L in enumerate(layers):
+        src = getattr(L.mixer, "kv_from", None)
+        if src is not None:
+            o = layers[src].mixer if 0 <= src < i else None
+            if not isinstance(o, AttentionSpec) or o.kv_from is not None or (o.kv_heads, o.dim, o.vdim) != (L.mixer.kv_heads, L.mixer.dim, L.mixer.vdim):
+                raise ValueError(f"layer {i}: kv_from {src} must name an earlier attention layer with its own keys and values of the same shape")
+
+
+def nepudra_from_json(cfg: dict) -> HybridConfig:
+    """The Nepudra reading of config.json.  Layer types: "general_delta" (mixer.{heads, dim}: key and value size are both dim),
+    "attention" (mixer.{heads, kv_heads, dim, vdim, scale, softcap, q_temp.{coef, every}, kv_from}: biased projections, no rotation, causal)
+    and "attention_2" (mixer.{heads, kv_heads, dim, vdim, scale, mask.size, rot.{dims, base, scaling}}: biased q / k / v, normed queries and
+    keys, rotary pairs half a span apart, sliding window); both attentions gate every head's output.  mlp: null or {kind: dense, ff}."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        kind, mx, mlp = L["type"], L["mixer"], L.get("mlp")
+        src = None if mx.get("kv_from") is None else int(mx["kv_from"])
+        if kind == "general_delta":
+            spec, kind = DeltaRuleSpec(heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx["dim"])), "delta_rule"
+        elif kind == "attention":
+            qt = mx.get("q_temp")
+            spec = AttentionSpec(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]), vdim=int(mx["vdim"]),
+                                 scale=float(mx["scale"]), kv_from=src, softcap=float(mx.get("softcap") or 0.0),
+                                 q_temp=(float(qt["coef"]), int(qt["every"])) if qt else None, bias=True, out_bias=True, out_gate=True)
+        elif kind == "attention_2":
+            mask = mx.get("mask") or {}
+            spec = AttentionSpec(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]), vdim=int(mx["vdim"]),
+                                 scale=float(mx["scale"]), rot=RotarySpec.from_json(mx.get("rot"), "halves"), kv_from=src,
+                                 window=int(mask.get("size", 0) or 0), qk_norm=True, bias=True, out_gate=True)
+            kind = "attention"
+        else:
+            raise NotImplementedError(f"layer {i}: mixer type {kind!r}")
+        if mlp is not None and mlp.get("kind", "dense") != "dense":
+            raise NotImplementedError(f"layer {i}: mlp kind {mlp.get('kind')!r}")
+        layers.append(HybridLayerSpec(kind, spec, None if mlp is None else int(mlp["ff"]), "gelu_tanh"))
+    _check_kv_from(layers)
+    bg = (cfg.get("embedding") or {}).get("bigram")
+    return HybridConfig(name=str(cfg["architecture"]), vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=layers, eps=float(cfg["norm"]["eps"]),
+                        norm_offset=0.0, sequential=True, scalar_norm=True, depth_mix=True,
+                        bigram=BigramSpec(int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"])) if bg else None)
+
+
+_READERS = {"nufalorn": HybridConfig.nufalorn_from_json, "pokepel": HybridConfig.pokepel_from_json, "nepudra": nepudra_from_json}
 
 
 class HybridModel:
@@ -143,9 +198,25 @@ class HybridModel:
         def sub(prefix, names):
             return {n: get(prefix + n) for n in names}
 
+        def norm_w(name):                             # a norm with one gain is run as a norm whose weight repeats it over the channels
+            t = get(name)
+            return t.reshape(1).expand(cfg.width).contiguous() if cfg.scalar_norm else t
+
         self.embed = get("embed")
         self.head = get("head")
-        self.final_norm = get("final.norm")
+        self.final_norm = norm_w("final.norm")
+        self.bigram = None
+        if cfg.bigram is not None:
+            self.bigram = get("bigram")
+            if self.bigram.shape != (cfg.bigram.buckets + 1, cfg.width):
+                raise ValueError(f"bigram table {tuple(self.bigram.shape)} for {cfg.bigram.buckets} buckets of width {cfg.width}")
+        self.depth_coef = []                             # layer i: fp32 [i + 2] weights over X_0 .. X_(i+1)
+        if cfg.depth_mix:
+            for i in range(len(cfg.layers)):
+                c = tensors[f"l{i}.dwa"].to(device=self.device, dtype=torch.float32).contiguous()
+                if c.numel() != i + 2:
+                    raise ValueError(f"l{i}.dwa has {c.numel()} weights for {i + 2} results")
+                self.depth_coef.append(c)
         if self.embed.shape != (cfg.vocab, cfg.width) or self.head.shape != (cfg.vocab, cfg.width):
             raise ValueError(f"embed {tuple(self.embed.shape)} / head {tuple(self.head.shape)} against vocab {cfg.vocab} width {cfg.width}")
         self.layers = []
@@ -153,8 +224,13 @@ class HybridModel:
         for i, L in enumerate(cfg.layers):
             p = f"l{i}."
             if L.kind == "attention":
-                names = ["q", "o"] + (["k", "v"] if L.mixer.kv_from is None else [])
-                mixer = PagedChunkAttention(L.mixer, sub(p + "mix.", names), cfg.eps, page, self.device)
+                a, own = L.mixer, L.mixer.kv_from is None
+                names = ["q", "o"] + (["k", "v"] if own else []) + (["g"] if a.out_gate else []) + (["o.b"] if a.out_bias else [])
+                names += (["q.b"] + (["k.b", "v.b"] if own else [])) if a.bias else []
+                names += (["q.norm"] + (["k.norm"] if own else [])) if a.qk_norm else []
+                mixer = PagedChunkAttention(a, sub(p + "mix.", names), cfg.eps, page, self.device)
+            elif L.kind == "delta_rule":
+                mixer = GeneralizedDeltaRule(L.mixer, sub(p + "mix.", ["r", "k", "v", "a", "a.b", "g", "w1", "w2", "w0", "norm", "o"]), cfg.eps)
             elif L.kind == "latent_attention":
                 mixer = LatentAttention(L.mixer, sub(p + "mix.", ["q", "dkv", "dkv.norm", "uk", "uv", "sink", "g", "o"]), cfg.eps, page, self.device)
             elif L.kind == "retention":
@@ -187,7 +263,7 @@ class HybridModel:
                     rw = torch.cat([mlp.w_router, torch.zeros((-E) % 4, cfg.width, dtype=dtype, device=self.device)], 0)
                     gate_w = torch.cat([gate_w, rw], 0).contiguous()
                     gate_b = torch.cat([gate_b, torch.zeros(rw.shape[0], dtype=dtype, device=self.device)], 0).contiguous()
-            n2 = get(p + "norm2") if mlp is not None and not cfg.shared_norm else None
+            n2 = norm_w(p + "norm2") if mlp is not None and not cfg.shared_norm else None
             if gate_w is not None and cfg.shared_norm and isinstance(mixer, (LatentAttention, Retention)):
                 # every projection of the layer's one normed input in ONE linear: [mixer inputs (padded to 4 columns) | gates | router]
                 pad = (-mixer.w_in.shape[0]) % 4
@@ -196,8 +272,8 @@ class HybridModel:
                 gate_b = torch.cat([torch.zeros(mixer.w_in.shape[0] + pad, dtype=dtype, device=self.device), gate_b], 0).contiguous()
                 gate_w = torch.cat([mixer.w_in, zrow, gate_w], 0).contiguous()
                 mixer.w_in = None                      # lives on as the leading rows of the shared weight
-            self.layers.append((L, mixer, mlp, get(p + "norm1"), n2, gate_w, gate_b))
-        self.has_state = any(L.kind not in ("attention", "latent_attention") for L in cfg.layers)
+            self.layers.append((L, mixer, mlp, norm_w(p + "norm1"), n2, gate_w, gate_b))
+        self.has_state = any(L.kind not in ("attention", "latent_attention") for L in cfg.layers) or cfg.bigram is not None
 
     # ---- what an engine has to allocate
     def cache_layout(self):
@@ -205,7 +281,7 @@ class HybridModel:
         out = []
         for L, mixer, *_ in self.layers:
             if L.kind == "attention":
-                out.append(("kv",) + mixer.cache_shapes() if mixer.owns_cache else ("kv_from", L.mixer.kv_from))
+                out.append((("kv",) + mixer.cache_shapes()) if mixer.owns_cache else ("kv_from", L.mixer.kv_from))
             elif L.kind == "latent_attention":
                 out.append(("latent", mixer.cache_shape()))
             else:
@@ -232,6 +308,8 @@ class HybridModel:
         """fp32 logits [len(batch.want), vocab] of the wanted rows; the caches of every row's sequence are advanced.  collect: receives
         the residual stream after every layer (debugging / tests; costs one extra norm launch per layer)."""
         cfg = self.cfg
+        if cfg.sequential:
+            return self._forward_sequential(batch, caches, collect)
         x = hops.embed(batch.tokens, self.embed)
         a = b = g = None
         shared = self.n_mix
@@ -265,6 +343,36 @@ class HybridModel:
             a = b = g = None
         hf, _ = hops.residual_norm(x, a, b, cfg.residual_mult, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset, rows=batch.want, gate=g)
         return hops.dense_linear(hf, self.head, out_dtype=torch.float32, softcap=cfg.logit_softcap)
+
+
+    def _forward_sequential(self, batch: StepBatch, caches, collect: Optional[list]) -> torch.Tensor:
+        """The step of a member whose two sublayers follow each other: x <- x + mixer(norm1 x), x <- x + mlp(norm2 x).  With depth_mix the
+        results X_1 .. of all layers and the embedding output X_0 are kept for the step, and the end of layer i replaces the stream by
+        sum_j dwa_i[j] X_j, fused with the last residual update and the next norm."""
+        cfg, T = self.cfg, batch.tokens.numel()
+        n_layers = len(self.layers)
+        stack = torch.empty(n_layers + 1 if cfg.depth_mix else 0, T, cfg.width, dtype=torch.float32, device=self.device)
+        bg = cfg.bigram
+        x = hops.embed(batch.tokens, self.embed, prev=batch.prev if bg else None, bigram=self.bigram, mul_prev=bg.mul_prev if bg else 0,
+                       mul_cur=bg.mul_cur if bg else 0, copy=stack[0] if cfg.depth_mix else None)
+        h1, _ = hops.residual_norm(x, None, None, 1.0, self.layers[0][3], None, cfg.eps, weight_offset=cfg.norm_offset)
+        for i, ((L, mixer, mlp, n1, n2, _gw, _gb), cache) in enumerate(zip(self.layers, caches)):
+            a = mixer.forward(h1, batch, *cache) if isinstance(cache, tuple) else mixer.forward(h1, batch, cache)
+            if mlp is not None:
+                h2, _ = hops.residual_norm(x, a, None, 1.0, n2, None, cfg.eps, weight_offset=cfg.norm_offset)
+                a = mlp.forward(h2)
+            last = i + 1 == n_layers
+            nw = self.final_norm if last else self.layers[i + 1][3]
+            rows = batch.want if last and collect is None else None
+            if cfg.depth_mix:
+                h1 = hops.depth_mix_norm(x, a, stack, i + 1, self.depth_coef[i], nw, cfg.eps, weight_offset=cfg.norm_offset, rows=rows)
+            else:
+                h1, _ = hops.residual_norm(x, a, None, 1.0, nw, None, cfg.eps, weight_offset=cfg.norm_offset, rows=rows)
+            if collect is not None:
+                collect.append(x.clone())
+        if collect is not None:
+            h1, _ = hops.residual_norm(x, None, None, 1.0, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset, rows=batch.want)
+        return hops.dense_linear(h1, self.head, out_dtype=torch.float32, softcap=cfg.logit_softcap)
 
 
 def load_hybrid_checkpoint(path: str, dtype: torch.dtype, device, page: int = 64) -> HybridModel:

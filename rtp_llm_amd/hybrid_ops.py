@@ -9,8 +9,8 @@ import torch
 
 from . import _C
 
-ACT_NONE, ACT_RELU, ACT_SILU = 0, 1, 2
-ACTIVATIONS = {"none": ACT_NONE, "relu": ACT_RELU, "silu": ACT_SILU}
+ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU_TANH, ACT_TANH = 0, 1, 2, 3, 4
+ACTIVATIONS = {"none": ACT_NONE, "relu": ACT_RELU, "silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH, "tanh": ACT_TANH}
 SCAN_HGRN2, SCAN_GLA, SCAN_FIXED = 0, 1, 2
 LAYOUTS = {"interleaved": 0, "halves": 1}
 
@@ -48,7 +48,8 @@ def _rows(t: torch.Tensor, name: str) -> int:
 def dense_linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, *, out_dtype: Optional[torch.dtype] = None,
                  gated: bool = False, act: int = ACT_NONE, softcap: float = 0.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x @ w.T (+ bias) for w [N, K] in checkpoint layout.  gated: w holds groups of 32 gate rows followed by the 32 up rows of the
-    same channels and y [M, N / 2] = act(gate) * up.  out_dtype float32 keeps the accumulator; softcap > 0 applies cap * tanh(y / cap)."""
+    same channels and y [M, N / 2] = act(gate) * up; without `gated`, act applies to the plain output.  out_dtype float32 keeps the accumulator;
+    softcap > 0 applies cap * tanh(y / cap)."""
     _dev(x, w.dtype, "dense_linear.x"); _dev(w, w.dtype, "dense_linear.w")
     ldx = _rows(x, "dense_linear.x")
     M, K = x.shape
@@ -91,15 +92,55 @@ def group_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.stack([gate.view(ff // 32, 32, K), up.view(ff // 32, 32, K)], dim=1).reshape(2 * ff, K).contiguous()
 
 
-def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """fp32 stream rows [T, W] of the token ids."""
+def embed(ids: torch.Tensor, table: torch.Tensor, *, prev: Optional[torch.Tensor] = None, bigram: Optional[torch.Tensor] = None, mul_prev: int = 0,
+          mul_cur: int = 0, copy: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 stream rows [T, W] of the token ids.  bigram [buckets + 1, W] with prev (int32 [T]: the token before each row in its sequence, -1 for
+    a sequence's first token): the row (prev * mul_prev + id * mul_cur) mod buckets of the table is added (its last row for a first token).
+    copy: an fp32 [T, W] tensor that receives the same rows."""
     _dev(ids, torch.int32, "embed.ids")
-    T = ids.numel()
-    out = torch.empty(T, table.shape[1], dtype=torch.float32, device=table.device)
+    T, W = ids.numel(), table.shape[1]
+    out = torch.empty(T, W, dtype=torch.float32, device=table.device)
+    buckets = 0
+    if bigram is not None:
+        _dev(bigram, table.dtype, "embed.bigram"); _dev(prev, torch.int32, "embed.prev")
+        buckets = bigram.shape[0] - 1
+        if bigram.dim() != 2 or bigram.shape[1] != W or buckets < 1 or prev.numel() != T or not bigram.is_contiguous():
+            raise _C.Mi355Error(f"embed: bigram table {tuple(bigram.shape)} / prev {tuple(prev.shape)} for {T} rows of {W}")
+    if copy is not None:
+        _dev(copy, torch.float32, "embed.copy")
+        if copy.shape != (T, W) or not copy.is_contiguous():
+            raise _C.Mi355Error(f"embed: copy {tuple(copy.shape)} for [{T}, {W}]")
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_embed(ids.data_ptr(), T, table.data_ptr(), table.shape[1], table.shape[0], out.data_ptr(),
-                                                       act_code(table.dtype), _stream()), "hy_embed")
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_embed_bigram(ids.data_ptr(), T, table.data_ptr(), W, table.shape[0], out.data_ptr(), _p(prev), _p(bigram),
+                                                              buckets, int(mul_prev), int(mul_cur), _p(copy), act_code(table.dtype), _stream()), "hy_embed")
     return out
+
+
+def depth_mix_norm(x: torch.Tensor, a: Optional[torch.Tensor], stack: torch.Tensor, n: int, coef: torch.Tensor, w1: Optional[torch.Tensor], eps: float, *,
+                   weight_offset: float = 0.0, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """The end of layer n - 1 of a stack whose layers read a weighted average of ALL earlier results: stack[n] <- x + a (the layer's own result; a may
+    be None), x <- sum_{j <= n} coef[j] * stack[j] (fp32, in the order of j), then the RMS norm of the new rows under w1 -> h1 in the weight's dtype
+    (None without w1).  stack fp32 [>= n + 1, T, W] holds the embedding output and the results of the layers before; coef fp32 [n + 1] on the device.
+    rows (int32): only these rows are formed and nothing is written back (the final norm of the rows whose logits are wanted)."""
+    _dev(x, torch.float32, "depth_mix_norm.x"); _dev(stack, torch.float32, "depth_mix_norm.stack"); _dev(coef, torch.float32, "depth_mix_norm.coef")
+    T, W = x.shape
+    if stack.dim() != 3 or stack.shape[1:] != (T, W) or stack.shape[0] < n + 1 or not stack.is_contiguous() or not x.is_contiguous() or coef.numel() != n + 1:
+        raise _C.Mi355Error(f"depth_mix_norm: stack {tuple(stack.shape)} coef {tuple(coef.shape)} for entry {n} of a stream {tuple(x.shape)}")
+    if a is not None:
+        _dev(a, torch.float32, "depth_mix_norm.a")
+        if a.shape != x.shape or not a.is_contiguous():
+            raise _C.Mi355Error(f"depth_mix_norm.a: {tuple(a.shape)} against the stream {tuple(x.shape)}")
+    if rows is not None:
+        _dev(rows, torch.int32, "depth_mix_norm.rows")
+    if w1 is not None and w1.numel() != W:
+        raise _C.Mi355Error(f"depth_mix_norm: weight {tuple(w1.shape)} for width {W}")
+    cnt = T if rows is None else rows.numel()
+    h1 = torch.empty(cnt, W, dtype=w1.dtype, device=x.device) if w1 is not None else None
+    if cnt:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_depth_mix_norm(x.data_ptr(), _p(a), stack.data_ptr(), T * W, n, coef.data_ptr(), _p(rows), cnt, W, _p(w1),
+                                                                float(weight_offset), float(eps), _p(h1), act_code(w1.dtype if w1 is not None else torch.float32),
+                                                                _stream()), "hy_depth_mix_norm")
+    return h1
 
 
 class MoeSum:
@@ -156,18 +197,26 @@ def attn_geometry(heads, kv_heads, dim, vdim, rot_dims, rot_layout, v_layout, pa
 
 
 def attn_prep(qkv: torch.Tensor, koff: int, voff: int, geom, kfreq, vfreq, v_norm: bool, eps: float, pos, seq, block_table,
-              kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor]):
+              kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], *, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
+              mag: float = 1.0, q_temp=None, cache_dtype: Optional[torch.dtype] = None):
     """Rotate the query heads of qkv (fp32 [T, ld], in place); with caches: rotate the keys, unit-norm and rotate the values, and write both
-    to their pages."""
+    to their pages.  q_norm / k_norm ([dim] in the cache dtype): queries / keys are brought to unit RMS per head and multiplied by the weight
+    before the rotation; mag multiplies cos and sin; q_temp = (coef, every): queries are multiplied by 1 + coef ln(floor((p + 1) / every) + 1)."""
     _dev(qkv, torch.float32, "attn_prep.qkv")
     ld = _rows(qkv, "attn_prep.qkv")
     T = qkv.shape[0]
     if not T:
         return
-    dt = kcache.dtype if kcache is not None else torch.float32
-    _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_prep(qkv.data_ptr(), ld, koff, voff, geom, _p(kfreq), _p(vfreq), 1 if v_norm else 0, float(eps),
-                                                       pos.data_ptr(), seq.data_ptr(), _p(block_table), T, _p(kcache), _p(vcache), act_code(dt),
-                                                       _stream()), "hy_attn_prep")
+    dt = kcache.dtype if kcache is not None else (cache_dtype or torch.float32)
+    for t, nm in ((q_norm, "q_norm"), (k_norm, "k_norm")):
+        if t is not None:
+            _dev(t, dt, "attn_prep." + nm)
+            if t.numel() != geom[2] or not t.is_contiguous():
+                raise _C.Mi355Error(f"attn_prep.{nm}: {tuple(t.shape)} for heads of {geom[2]}")
+    coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp else (0.0, 1)
+    _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_prep_ex(qkv.data_ptr(), ld, koff, voff, geom, _p(kfreq), _p(vfreq), 1 if v_norm else 0, float(eps),
+                                                          pos.data_ptr(), seq.data_ptr(), _p(block_table), T, _p(kcache), _p(vcache), _p(q_norm), _p(k_norm),
+                                                          float(mag), coef, every, act_code(dt), _stream()), "hy_attn_prep")
 
 
 def _sink(sink: Optional[torch.Tensor], heads: int):
@@ -178,24 +227,40 @@ def _sink(sink: Optional[torch.Tensor], heads: int):
     return _p(sink)
 
 
+def _ogate(gate: Optional[torch.Tensor], T: int, heads: int, name: str):
+    if gate is None:
+        return None, 0
+    _dev(gate, torch.float32, name)
+    ld = _rows(gate, name)
+    if gate.shape != (T, heads):
+        raise _C.Mi355Error(f"{name}: {tuple(gate.shape)} for {T} rows of {heads} heads")
+    return gate.data_ptr(), ld
+
+
 def attn_rows(q: torch.Tensor, scale: float, geom, chunk: int, sink: Optional[torch.Tensor], vfreq, pos, seq, block_table, kcache, vcache,
-              heads: int, vdim: int):
+              heads: int, vdim: int, *, window: int = 0, softcap: float = 0.0, out_gate: Optional[torch.Tensor] = None):
     """Attention of every row over its sequence's pages -> [T, heads * vdim] in the cache dtype.  sink: fp32 [heads] or None; exp(sink[h])
     joins head h's softmax denominator.  Few rows over long block tables (decode steps) are dealt over several blocks per (row, head) whose
-    partial sums a second launch merges; the count depends on the rows and the table's width only."""
+    partial sums a second launch merges; the count depends on the rows and the table's width only.  window > 0: a row at position i sees
+    the keys j with 0 <= i - j < window; softcap > 0: cap * tanh(score / cap) on the scaled scores; out_gate fp32 [T, heads] (a column slice is
+    fine): head h of a row is multiplied by the sigmoid of its entry."""
     _dev(q, torch.float32, "attn_rows.q")
     T = q.shape[0]
     out = torch.empty(T, heads * vdim, dtype=kcache.dtype, device=q.device)
     splits, parts = 1, None
+    gp, ldg = _ogate(out_gate, T, heads, "attn_rows.out_gate")
     if chunk == 0 and T * heads <= 2048:                   # sixteen waves per block: one 64-key tile per wave and block where the chip has room
         tiles = (block_table.shape[1] * geom[7] + 63) // 64
+        if window > 0:
+            tiles = min(tiles, (window + 63) // 64 + 1)
         splits = max(1, min(16, (tiles + 15) // 16, 1024 // (T * heads)))
         if splits > 1:
             parts = torch.empty(T * heads * splits * (vdim + 2), dtype=torch.float32, device=q.device)
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_rows(q.data_ptr(), _rows(q, "attn_rows.q"), float(scale), geom, int(chunk), _sink(sink, heads), _p(vfreq),
-                                                           pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), T, kcache.data_ptr(), vcache.data_ptr(),
-                                                           out.data_ptr(), splits, _p(parts), act_code(kcache.dtype), _stream()), "hy_attn_rows")
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_rows_ex(q.data_ptr(), _rows(q, "attn_rows.q"), float(scale), geom, int(chunk), _sink(sink, heads), _p(vfreq),
+                                                              pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), T, kcache.data_ptr(), vcache.data_ptr(),
+                                                              out.data_ptr(), splits, _p(parts), int(window), float(softcap), gp, ldg, act_code(kcache.dtype),
+                                                              _stream()), "hy_attn_rows")
     return out
 
 
@@ -205,17 +270,18 @@ def attn_tiles_supported(dtype: torch.dtype, dim: int, vdim: int, value_rot: boo
 
 
 def attn_tiles(q: torch.Tensor, scale: float, geom, chunk: int, sink: Optional[torch.Tensor], vfreq, pos, seq, block_table, tile_row0, tile_n, kcache, vcache,
-               heads: int, vdim: int):
+               heads: int, vdim: int, *, window: int = 0, softcap: float = 0.0, out_gate: Optional[torch.Tensor] = None):
     """attn_rows for prompt portions on the matrix cores: tile t = rows tile_row0[t] .. + tile_n[t] - 1 (at most 16 consecutive rows of one
     sequence); every row of the batch must lie in exactly one tile."""
     _dev(q, torch.float32, "attn_tiles.q"); _dev(tile_row0, torch.int32, "attn_tiles.tile_row0"); _dev(tile_n, torch.int32, "attn_tiles.tile_n")
     T = q.shape[0]
     out = torch.empty(T, heads * vdim, dtype=kcache.dtype, device=q.device)
+    gp, ldg = _ogate(out_gate, T, heads, "attn_tiles.out_gate")
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_tiles(q.data_ptr(), _rows(q, "attn_tiles.q"), float(scale), geom, int(chunk), _sink(sink, heads), _p(vfreq),
-                                                            pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), tile_row0.data_ptr(), tile_n.data_ptr(),
-                                                            tile_row0.numel(), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(),
-                                                            act_code(kcache.dtype), _stream()), "hy_attn_tiles")
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_tiles_ex(q.data_ptr(), _rows(q, "attn_tiles.q"), float(scale), geom, int(chunk), _sink(sink, heads), _p(vfreq),
+                                                               pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), tile_row0.data_ptr(), tile_n.data_ptr(),
+                                                               tile_row0.numel(), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(), int(window),
+                                                               float(softcap), gp, ldg, act_code(kcache.dtype), _stream()), "hy_attn_tiles")
     return out
 
 
@@ -234,18 +300,46 @@ def scan(mode: int, proj: torch.Tensor, qo: int, ko: int, vo: int, z: Optional[t
     return out
 
 
+def delta_scan(proj: torch.Tensor, ro: int, ko: int, vo: int, ao: int, z: torch.Tensor, decay_mult: float, unit_eps: float, heads: int, dim: int,
+               vdim: int, row_start, slot, first_pos, state: torch.Tensor) -> torch.Tensor:
+    """Generalized delta rule over the rows of every sequence: S <- diag(w) S - (a * u)(u^T S) + k v^T (both terms from the old state), o = S^T r,
+    with w = exp(-decay_mult * sigmoid(z)), a = sigmoid(proj[:, ao:]), u = k / sqrt(|k|^2 + unit_eps) per head; r, k (heads x dim) and v (heads x
+    vdim) are fp32 columns ro, ko, vo of proj, z fp32 [T, heads * dim].  Continues and leaves the fp32 state [slots, heads, dim, vdim] of each
+    sequence's slot -> fp32 [T, heads * vdim]."""
+    _dev(proj, torch.float32, "delta_scan.proj"); _dev(state, torch.float32, "delta_scan.state"); _dev(z, torch.float32, "delta_scan.z")
+    T = proj.shape[0]
+    ld, ldz = _rows(proj, "delta_scan.proj"), _rows(z, "delta_scan.z")
+    hd = heads * dim
+    if max(ro, ko, ao) + hd > proj.shape[1] or vo + heads * vdim > proj.shape[1] or z.shape != (T, hd) or state.shape[1:] != (heads, dim, vdim) or not state.is_contiguous():
+        raise _C.Mi355Error(f"delta_scan: proj {tuple(proj.shape)} z {tuple(z.shape)} state {tuple(state.shape)} for {heads} heads of {dim} x {vdim}")
+    out = torch.empty(T, heads * vdim, dtype=torch.float32, device=proj.device)
+    nseq = slot.numel()
+    if T and nseq:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_delta_scan(proj.data_ptr(), ld, ro, ko, vo, ao, z.data_ptr(), ldz, float(decay_mult), float(unit_eps), heads, dim,
+                                                            vdim, row_start.data_ptr(), slot.data_ptr(), first_pos.data_ptr(), nseq, state.data_ptr(),
+                                                            out.data_ptr(), _stream()), "hy_delta_scan")
+    return out
+
+
 def head_norm(o: torch.Tensor, heads: int, vdim: int, w: Optional[torch.Tensor], eps: float, gate: Optional[torch.Tensor] = None, goff: int = 0,
-              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """Per-head RMS norm of o (fp32 [T, heads * vdim]) under the shared weight w [vdim] (None: unit RMS only, output in `out_dtype`),
-    times silu(gate[:, goff:]) when a gate is given."""
+              out_dtype: Optional[torch.dtype] = None, gate_act: str = "silu") -> torch.Tensor:
+    """Per-head RMS norm of o (fp32 [T, heads * vdim]) under the weight w ([vdim] shared by the heads, or [heads * vdim]; None: unit RMS only,
+    output in `out_dtype`), times gate_act(gate[:, goff:]) ("silu" or "sigmoid") when a gate is given."""
     _dev(o, torch.float32, "head_norm.o")
     T = o.shape[0]
     dt = w.dtype if w is not None else out_dtype
     out = torch.empty(T, heads * vdim, dtype=dt, device=o.device)
+    per_head = 0
+    if w is not None:
+        if w.numel() not in (vdim, heads * vdim) or not w.is_contiguous():
+            raise _C.Mi355Error(f"head_norm: weight {tuple(w.shape)} for {heads} heads of {vdim}")
+        per_head = 1 if w.numel() == heads * vdim and heads > 1 else 0
+    if gate_act not in ("silu", "sigmoid"):
+        raise _C.Mi355Error(f"head_norm: gate activation {gate_act!r}")
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_head_norm(o.data_ptr(), T, heads, vdim, _p(w), float(eps), _p(gate),
-                                                           0 if gate is None else _rows(gate, "head_norm.gate"), goff, out.data_ptr(),
-                                                           act_code(dt), _stream()), "hy_head_norm")
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_head_norm_ex(o.data_ptr(), T, heads, vdim, _p(w), float(eps), _p(gate),
+                                                              0 if gate is None else _rows(gate, "head_norm.gate"), goff, out.data_ptr(), per_head,
+                                                              1 if gate_act == "sigmoid" else 0, act_code(dt), _stream()), "hy_head_norm")
     return out
 
 

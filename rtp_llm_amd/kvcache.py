@@ -110,10 +110,11 @@ class SlotPool(PagePool):
 
 
 class SequenceCache:
-    """What one live sequence holds: its pages (in position order), its state slot and the number of tokens already run."""
+    """What one live sequence holds: its pages (in position order), its state slot, the number of tokens already run and the last of them
+    (-1 before the first: models whose embedding looks at the previous token continue from it)."""
 
     def __init__(self, slot: int):
-        self.pages, self.slot, self.length = [], slot, 0
+        self.pages, self.slot, self.length, self.last_token = [], slot, 0, -1
 
 
 class CacheManager:
@@ -151,8 +152,11 @@ class CacheManager:
             self._promised[sid] = max(0, self._promised[sid] - need)
         return sc
 
-    def advance(self, sid, new_tokens: int):
-        self.live[sid].length += new_tokens
+    def advance(self, sid, new_tokens: int, last_token: Optional[int] = None):
+        sc = self.live[sid]
+        sc.length += new_tokens
+        if last_token is not None:
+            sc.last_token = int(last_token)
 
     def release(self, sid):
         sc = self.live.pop(sid)

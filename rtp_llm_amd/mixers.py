@@ -4,7 +4,13 @@
     mask that is causal inside blocks of `chunk` positions (0: plain causal), an optional softmax sink (one added to the denominator),
     optional unit-normed values and optional value rotation (values are turned by their own position when cached and the head output
     is turned back by the query's position, so a value enters the sum turned by the distance).  A layer may read the cache that an
-    earlier layer with the same geometry wrote (`kv_from`) and then has no key / value projections.
+    earlier layer with the same geometry wrote (`kv_from`) and then has no key / value projections.  Further options, each off by default:
+    a sliding window instead of the block mask, a tanh cap on the scaled scores, a temperature on the queries that grows with the
+    logarithm of the position, RMS-normed queries and keys under weights shared by the heads, YaRN-scaled rotary steps, biases on the
+    projections, and a sigmoid gate per head on the output.
+  * ``GeneralizedDeltaRule`` -- S_t = diag(w_t) S_(t-1) - (a_t * u_t)(u_t^T S_(t-1)) + k_t v_t^T, o_t = S_t^T r_t per head with the state in an
+    fp32 slot: a per-channel decay w from a low-rank projection, a per-channel removal rate a along the unit key u, heads brought to unit
+    RMS under a per-channel weight and gated by a sigmoid.
   * ``GatedLinearRecurrence`` -- S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head with the state in an fp32 slot, in the
     HGRN2 parametrisation (a = f, k = 1 - f with a lower-bounded forget gate f, q = silu) or the gated-linear-attention one
     (a = sigmoid(low-rank z)^(1/tau), q scaled by dim^-1/2, output gate silu(g)); per-head RMS norm of o, then the output projection.
@@ -67,6 +73,13 @@ class AttentionSpec:
     value_rot: bool = False
     value_layout: str = "interleaved"
     kv_from: Optional[int] = None
+    window: int = 0                      # > 0 (chunk must be 0): position i sees the keys j with 0 <= i - j < window
+    softcap: float = 0.0                 # > 0: scaled scores become softcap * tanh(score / softcap)
+    q_temp: Optional[tuple] = None       # (coef, every): queries at position p are multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)
+    qk_norm: bool = False                # queries and keys are RMS-normed per head under weights [dim] shared by the heads, before the rotation
+    bias: bool = False                   # the q, k, v projections have biases
+    out_bias: bool = False               # the output projection has a bias
+    out_gate: bool = False               # head h's output is multiplied by sigmoid(W_g x)_h, one number per head
 
 
 @dataclass
@@ -76,6 +89,15 @@ class RecurrenceSpec:
     dim: int
     vdim: int
     tau: float = 1.0
+
+
+@dataclass
+class DeltaRuleSpec:
+    heads: int
+    dim: int                             # key channels per head
+    vdim: int                            # value channels per head
+    decay_mult: float = math.exp(-0.5)   # w = exp(-decay_mult * sigmoid(.)): the decay of a channel stays above exp(-decay_mult)
+    unit_eps: float = 1e-6               # u = k / sqrt(|k|^2 + unit_eps)
 
 
 @dataclass
@@ -93,6 +115,7 @@ class StepBatch:
     want: torch.Tensor                   # rows whose logits are computed
     tile_row0: Optional[torch.Tensor] = None   # tiles of at most 16 consecutive rows of one sequence covering every row: first row ...
     tile_n: Optional[torch.Tensor] = None      # ... and row count (the matrix-core attention for prompt portions works on them)
+    prev: Optional[torch.Tensor] = None        # the token before each row in its sequence (-1 for a sequence's first token): bigram embeddings
     host: Optional[torch.Tensor] = None        # the pinned buffer all index fields were uploaded from (one copy per step)
 
 
@@ -117,18 +140,32 @@ def rotary_steps(n_pairs: int, span: int, base: float, device) -> torch.Tensor:
 
 
 class PagedChunkAttention:
+    """weights: q [H dim, W], k [G dim, W], v [G vdim, W] (absent with kv_from), o [W, H vdim]; by option q.b / k.b / v.b / o.b, q.norm / k.norm [dim],
+    g [H, W].  Every projection of the input (q | k | v | gate) is one linear."""
+
     def __init__(self, spec: AttentionSpec, weights: Dict[str, torch.Tensor], eps: float, page: int, device):
         s = self.spec = spec
         self.eps, self.page = eps, page
         if s.heads % s.kv_heads:
             raise ValueError(f"attention: {s.heads} query heads over {s.kv_heads} key/value heads")
+        if s.window and s.chunk:
+            raise ValueError("attention: a sliding window and a block mask exclude each other")
         self.owns_cache = s.kv_from is None
-        parts = [weights["q"]] + ([weights["k"], weights["v"]] if self.owns_cache else [])
+        names = ["q"] + (["k", "v"] if self.owns_cache else [])
+        parts = [weights[n] for n in names] + ([weights["g"]] if s.out_gate else [])
         self.w_in = torch.cat(parts, 0).contiguous()
+        self.b_in = None
+        if s.bias:
+            zero = [torch.zeros(s.heads, dtype=self.w_in.dtype, device=self.w_in.device)] if s.out_gate else []
+            self.b_in = torch.cat([weights[n + ".b"] for n in names] + zero, 0).contiguous()
         self.w_o = weights["o"].contiguous()
+        self.b_o = weights["o.b"].contiguous() if s.out_bias else None
         self.koff, self.voff = s.heads * s.dim, (s.heads + s.kv_heads) * s.dim
+        self.goff = s.heads * s.dim + ((s.kv_heads * (s.dim + s.vdim)) if self.owns_cache else 0)
+        self.q_norm = weights["q.norm"].contiguous() if s.qk_norm else None
+        self.k_norm = weights["k.norm"].contiguous() if s.qk_norm and self.owns_cache else None
         rot = s.rot
-        self.kfreq = rotary_steps(rot.dims // 2, rot.dims, rot.base, device) if rot and rot.dims else None
+        self.kfreq, self.mag = rotary_table(rot, device) if rot and rot.dims else (None, 1.0)
         self.vfreq = rotary_steps(s.vdim // 2, s.vdim, rot.base, device) if s.value_rot and rot else None
         self._geom = None
         self.use_tiles = True
@@ -152,18 +189,55 @@ class PagedChunkAttention:
     def forward(self, h: torch.Tensor, batch: StepBatch, kcache: torch.Tensor, vcache: torch.Tensor) -> torch.Tensor:
         s = self.spec
         geom = self.geometry(batch.block_table.shape[1], kcache.shape[0])
-        qkv = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
+        qkv = hops.dense_linear(h, self.w_in, self.b_in, out_dtype=torch.float32)
         write = self.owns_cache
         hops.attn_prep(qkv, self.koff, self.voff, geom, self.kfreq, self.vfreq, s.value_norm, self.eps, batch.pos, batch.seq, batch.block_table,
-                       kcache if write else None, vcache if write else None)
+                       kcache if write else None, vcache if write else None, q_norm=self.q_norm, k_norm=self.k_norm, mag=self.mag, q_temp=s.q_temp,
+                       cache_dtype=kcache.dtype)
         T = qkv.shape[0]
+        extra = dict(window=s.window, softcap=s.softcap, out_gate=qkv[:, self.goff:self.goff + s.heads] if s.out_gate else None)
         # prompt portions (tiles mostly full) go to the matrix-core kernel, decode rows to the one that spreads a row's keys over four waves
         if (self.use_tiles and batch.tile_row0 is not None and batch.tile_row0.numel() * 4 <= T
                 and hops.attn_tiles_supported(kcache.dtype, s.dim, s.vdim, self.vfreq is not None, hops.LAYOUTS[s.value_layout])):
             o = hops.attn_tiles(qkv, s.scale, geom, s.chunk, self.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, batch.tile_row0, batch.tile_n,
-                                kcache, vcache, s.heads, s.vdim)
+                                kcache, vcache, s.heads, s.vdim, **extra)
         else:
-            o = hops.attn_rows(qkv, s.scale, geom, s.chunk, self.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, kcache, vcache, s.heads, s.vdim)
+            o = hops.attn_rows(qkv, s.scale, geom, s.chunk, self.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, kcache, vcache, s.heads, s.vdim,
+                               **extra)
+        return hops.dense_linear(o, self.w_o, self.b_o, out_dtype=torch.float32)
+
+
+class GeneralizedDeltaRule:
+    """weights: r, k, a [H dim, W], v, g [H vdim, W], a.b [H dim], w1 [rank, W], w2 [H dim, rank], w0 [H dim], norm [H vdim], o [W, H vdim].
+    One linear gives r | k | v | a (+ bias) | g in fp32; the decay's pre-activation is the low-rank pair w2 tanh(w1 x) + w0.  Decay, removal
+    rate, unit key, state and update are fp32 (hybrid_ops.delta_scan); the heads are brought to unit RMS, multiplied by `norm` and by
+    sigmoid(g), then projected."""
+
+    def __init__(self, spec: DeltaRuleSpec, weights: Dict[str, torch.Tensor], eps: float):
+        s = self.spec = spec
+        self.eps = eps
+        hd, hv = s.heads * s.dim, s.heads * s.vdim
+        for n, shape in (("r", hd), ("k", hd), ("a", hd), ("v", hv), ("g", hv), ("w2", hd)):
+            if weights[n].shape[0] != shape:
+                raise ValueError(f"delta rule: weight {n} {tuple(weights[n].shape)} for {s.heads} heads of {s.dim} x {s.vdim}")
+        self.w_in = torch.cat([weights[n] for n in ("r", "k", "v", "a", "g")], 0).contiguous()
+        z = lambda n: torch.zeros(n, dtype=self.w_in.dtype, device=self.w_in.device)
+        self.b_in = torch.cat([z(2 * hd + hv), weights["a.b"], z(hv)], 0).contiguous()
+        self.ro, self.ko, self.vo, self.ao, self.go = 0, hd, 2 * hd, 2 * hd + hv, 3 * hd + hv
+        self.w_w1, self.w_w2, self.b_w = weights["w1"].contiguous(), weights["w2"].contiguous(), weights["w0"].contiguous()
+        self.norm, self.w_o = weights["norm"].contiguous(), weights["o"].contiguous()
+
+    def state_shape(self):
+        s = self.spec
+        return (s.heads, s.dim, s.vdim)
+
+    def forward(self, h: torch.Tensor, batch: StepBatch, state: torch.Tensor) -> torch.Tensor:
+        s = self.spec
+        proj = hops.dense_linear(h, self.w_in, self.b_in, out_dtype=torch.float32)
+        z = hops.dense_linear(hops.dense_linear(h, self.w_w1, act=hops.ACT_TANH), self.w_w2, self.b_w, out_dtype=torch.float32)
+        o = hops.delta_scan(proj, self.ro, self.ko, self.vo, self.ao, z, s.decay_mult, s.unit_eps, s.heads, s.dim, s.vdim,
+                            batch.row_start, batch.slot, batch.first_pos, state)
+        o = hops.head_norm(o, s.heads, s.vdim, self.norm, self.eps, proj, self.go, gate_act="sigmoid")
         return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
 
 

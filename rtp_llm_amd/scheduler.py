@@ -50,16 +50,16 @@ class ServingEngine:
     # ------------------------------------------------------------------ the step function
     def build_batch(self, entries: Sequence[Tuple[object, Sequence[int], Sequence[int]]]) -> StepBatch:
         """entries: (sequence id, its next tokens, indices among them whose logits are wanted).  Admits new sequences and takes pages."""
-        tokens, pos, seq, row_start, slot, first, want, tables = [], [], [], [0], [], [], [], []
+        tokens, pos, seq, row_start, slot, first, want, tables, prev = [], [], [], [0], [], [], [], [], []
         seen, admitted = set(), []
         try:
-            return self._build(entries, tokens, pos, seq, row_start, slot, first, want, tables, seen, admitted)
+            return self._build(entries, tokens, pos, seq, row_start, slot, first, want, tables, seen, admitted, prev)
         except Exception:
             for sid in admitted:                      # a step that cannot run leaves no half-admitted sequence behind
                 self.cache.release(sid)
             raise
 
-    def _build(self, entries, tokens, pos, seq, row_start, slot, first, want, tables, seen, admitted):
+    def _build(self, entries, tokens, pos, seq, row_start, slot, first, want, tables, seen, admitted, prev):
         for sid, toks, wants in entries:
             if sid in seen:
                 raise ValueError(f"sequence {sid!r} appears twice in one step")
@@ -73,6 +73,7 @@ class ServingEngine:
             s = len(slot)
             base = len(tokens)
             tokens += [int(t) for t in toks]
+            prev += [sc.last_token if sc.length else -1] + [int(t) for t in toks[:-1]]
             pos += list(range(sc.length, sc.length + len(toks)))
             seq += [s] * len(toks)
             row_start.append(len(tokens))
@@ -92,7 +93,7 @@ class ServingEngine:
         for t in tables:
             bt += t + [0] * (width - len(t))
         # every index array of the step travels in ONE pinned int32 buffer and one copy; the fields are views into the device copy
-        parts = [tokens, pos, seq, row_start, slot, first, bt, want, t0, tn]
+        parts = [tokens, pos, seq, row_start, slot, first, bt, want, t0, tn, prev]
         offs = [0]
         for part in parts:
             offs.append(offs[-1] + (len(part) + 3) // 4 * 4)      # 16-byte aligned fields
@@ -125,7 +126,7 @@ class ServingEngine:
         else:
             logits = self.model.forward(batch, self.tensors, collect)
         for sid, toks, _ in entries:
-            self.cache.advance(sid, len(toks))
+            self.cache.advance(sid, len(toks), toks[-1])
         return logits if batch.want.numel() else None
 
     def _replay_decode(self, batch: StepBatch) -> torch.Tensor:
@@ -137,7 +138,7 @@ class ServingEngine:
             buf = torch.empty_like(batch.host, device=self.device)
             buf.copy_(batch.host)
             nseq, width = key
-            static = self.batch_views(buf, [nseq, nseq, nseq, nseq + 1, nseq, nseq, nseq * width, nseq, nseq, nseq], nseq, width)
+            static = self.batch_views(buf, [nseq, nseq, nseq, nseq + 1, nseq, nseq, nseq * width, nseq, nseq, nseq, nseq], nseq, width)
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
