@@ -6,6 +6,9 @@ against their rooflines (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 vector FM
 Nufalorn member at equal width, depth, heads, FFN width (active per token) and vocabulary, and Pokepel's kernels beside the like
 Nufalorn kernels against their rooflines.
 
+`--hybrid-design nepudra` does the same for the Nepudra member (delta-rule recurrence, capped causal and sliding-window attention with gated
+heads, bigram embedding, depth-averaged sequential layers).
+
 Output: one JSON line {"hybrid_bench": {size: {"hybrid": {...}, "qwen2": {...}, "kernels": [...]}}} (with --hybrid-design pokepel:
 {"pokepel": {...}, "nufalorn": {...}, "kernels": [...]})."""
 import json
@@ -131,6 +134,68 @@ def pokepel_weights(cfg, dev, seed=0):
     return w
 
 
+NEPUDRA_PATTERN = ["delta", "capped", "delta", "delta", "window", "shared", "delta", "delta"]
+
+
+def nepudra_config(s, window=1024):
+    """Width, depth, attention heads, FFN width and vocabulary of `s`; delta-rule layers with width / 64 heads of 64 key and value channels,
+    capped causal attention (one layer in eight reads the keys and values of the capped layer before it) and sliding-window attention
+    with normed, YaRN-rotated queries and keys over `window` positions; gelu-gated MLPs; a bigram table of 65521 buckets."""
+    layers, owner, hd = [], None, s["hd"]
+    for i in range(s["layers"]):
+        kind = NEPUDRA_PATTERN[i % len(NEPUDRA_PATTERN)]
+        mlp = {"kind": "dense", "ff": s["ff"]}
+        if kind == "delta":
+            layers.append({"type": "general_delta", "mixer": {"heads": s["width"] // 64, "dim": 64}, "mlp": mlp})
+        elif kind in ("capped", "shared"):
+            mx = {"heads": s["heads"], "kv_heads": s["kv"], "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 30.0, "q_temp": {"coef": 0.2, "every": 128}}
+            if kind == "shared":
+                mx["kv_from"] = owner
+            else:
+                owner = i
+            layers.append({"type": "attention", "mixer": mx, "mlp": mlp})
+        else:
+            mx = {"heads": s["heads"], "kv_heads": s["kv"], "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": window},
+                  "rot": {"base": 1e6, "dims": hd, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+            layers.append({"type": "attention_2", "mixer": mx, "mlp": mlp})
+    return {"architecture": "Nepudra", "layers": layers, "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 8191, "mul_cur": 131}}}
+
+
+def nepudra_weights(cfg, dev, seed=0, rank=64):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    W = cfg["width"]
+    lin = lambda o, i: (torch.randn(o, i, device=dev, generator=g) * i ** -0.5).bfloat16()
+    vec = lambda n, k=0.1, off=0.0: (torch.randn(n, device=dev, generator=g) * k + off).bfloat16()
+    one = lambda: torch.tensor(1.0, device=dev).bfloat16()
+    w = {"embed": torch.randn(cfg["vocab"], W, device=dev, generator=g).bfloat16(), "head": lin(cfg["vocab"], W), "final.norm": one(),
+         "bigram": (torch.randn(cfg["embedding"]["bigram"]["buckets"] + 1, W, device=dev, generator=g) * 0.5).bfloat16()}
+    for i, L in enumerate(cfg["layers"]):
+        p, mx = f"l{i}.", L["mixer"]
+        H, d = mx["heads"], mx["dim"]
+        w[p + "norm1"], w[p + "norm2"] = one(), one()
+        c = torch.full((i + 2,), 0.2 / (i + 1), device=dev)
+        c[-1] = 0.8
+        w[p + "dwa"] = c.bfloat16()
+        if L["type"] == "general_delta":
+            for n in ("r", "k", "v", "a", "g"):
+                w[p + "mix." + n] = lin(H * d, W)
+            w[p + "mix.a.b"], w[p + "mix.w1"], w[p + "mix.w2"], w[p + "mix.w0"] = vec(H * d, 0.5), lin(rank, W), lin(H * d, rank), vec(H * d, 1.0)
+            w[p + "mix.norm"], w[p + "mix.o"] = vec(H * d, 0.1, 1.0), lin(W, H * d)
+        else:
+            G, dv = mx["kv_heads"], mx["vdim"]
+            w[p + "mix.q"], w[p + "mix.q.b"], w[p + "mix.g"], w[p + "mix.o"] = lin(H * d, W), vec(H * d), lin(H, W), lin(W, H * dv)
+            if "kv_from" not in mx:
+                w[p + "mix.k"], w[p + "mix.k.b"], w[p + "mix.v"], w[p + "mix.v.b"] = lin(G * d, W), vec(G * d), lin(G * dv, W), vec(G * dv)
+            if L["type"] == "attention":
+                w[p + "mix.o.b"] = vec(W)
+            else:
+                w[p + "mix.q.norm"], w[p + "mix.k.norm"] = vec(d, 0.1, 1.0), vec(d, 0.1, 1.0)
+        ff = L["mlp"]["ff"]
+        w[p + "mlp.gate"], w[p + "mlp.up"], w[p + "mlp.down"] = lin(ff, W), lin(ff, W), lin(W, ff)
+    return w
+
+
 def timed(fn, reps=5, warm=2, graph=False):
     """Seconds per call.  graph: the calls are captured into one HIP graph and the replay is timed, so the figure is the kernels' own
     time and not the host's launch path (what a graph-replayed step pays)."""
@@ -165,8 +230,9 @@ def timed(fn, reps=5, warm=2, graph=False):
 def bench_hybrid_engine(s, dev, prompt, batch, steps, design="nufalorn"):
     from .hybrid import HybridConfig, HybridModel
     from .scheduler import ServingEngine
-    cfg = pokepel_config(s) if design == "pokepel" else hybrid_config(s)
-    model = HybridModel(HybridConfig.from_json(cfg), (pokepel_weights if design == "pokepel" else hybrid_weights)(cfg, dev), torch.bfloat16, dev)
+    make_cfg, make_w = {"pokepel": (pokepel_config, pokepel_weights), "nepudra": (nepudra_config, nepudra_weights)}.get(design, (hybrid_config, hybrid_weights))
+    cfg = make_cfg(s)
+    model = HybridModel(HybridConfig.from_json(cfg), make_w(cfg, dev), torch.bfloat16, dev)
     eng = ServingEngine(model, max_tokens=batch * (prompt + 8 * (steps + 3) + 128), max_seqs=batch, max_step_tokens=1 << 20)
     g = torch.Generator().manual_seed(1)
     toks = lambda n: torch.randint(0, s["vocab"], (n,), generator=g).tolist()
@@ -445,27 +511,152 @@ def kernel_table_pokepel(s, dev, prompt):
     return rows
 
 
+def kernel_table_nepudra(s, dev, prompt):
+    """Nepudra's kernels at this size beside the like kernels of the Nufalorn member, against max(bytes / HBM, flops / peak of the unit)."""
+    from . import hybrid_ops as hops
+    rows = []
+    timed_k = lambda fn: timed(fn, reps=10, warm=2, graph=True)
+    g = torch.Generator(device=dev).manual_seed(3)
+    bf = lambda *sh: torch.randn(*sh, device=dev, generator=g).bfloat16()
+    f32 = lambda *sh: torch.randn(*sh, device=dev, generator=g)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    W, H, G, hd, ff, L = s["width"], s["heads"], s["kv"], s["hd"], s["ff"], s["layers"]
+
+    def add(family, name, shape, t, nbytes, flops, peak):
+        roof = max(nbytes / HBM, flops / peak)
+        rows.append({"family": family, "kernel": name, "shape": shape, "us": round(t * 1e6, 1), "roofline_us": round(roof * 1e6, 2),
+                     "x_roofline": round(t / roof, 1)})
+
+    page, window = 64, 1024
+    nblk = (prompt + page - 1) // page + 1
+    bt = torch.arange(nblk, dtype=torch.int32, device=dev).reshape(1, nblk)
+    geom = hops.attn_geometry(H, G, hd, hd, hd, 1, 0, page, nblk, nblk)
+    ngeom = hops.attn_geometry(H, G, hd, hd, hd, 0, 0, page, nblk, nblk)
+    kc, vc = bf(nblk, G, page, hd), bf(nblk, G, page, hd)
+    vf = torch.ones(hd // 2, device=dev) * 1e-3
+    sink0 = torch.zeros(H, device=dev)
+    # attention: sliding window with gated heads against the block mask with sink and turned values; capped causal against plain causal
+    for T_, name in ((prompt, "prefill"), (1, "decode")):
+        pos = torch.arange(T_, dtype=torch.int32, device=dev) if T_ > 1 else i32([prompt - 1])
+        seq = torch.zeros(T_, dtype=torch.int32, device=dev)
+        q = f32(T_, H * hd + H)
+        og = q[:, H * hd:]
+        kw = float(sum(min(int(p) + 1, window) for p in pos.tolist()))
+        kb = float(sum(int(p) % window + 1 for p in pos.tolist()))
+        kc_ = float(sum(int(p) + 1 for p in pos.tolist()))
+        byt = lambda keys: min(prompt, keys) * G * hd * 2 * 2 + T_ * H * hd * 6
+        if T_ > 1:
+            t0 = torch.arange(0, T_, 16, dtype=torch.int32, device=dev)
+            tn = torch.full_like(t0, 16)
+            t = timed_k(lambda: hops.attn_tiles(q, hd ** -0.5, geom, 0, None, None, pos, seq, bt, t0, tn, kc, vc, H, hd, window=window, out_gate=og))
+            add("nepudra", f"attn_tiles prefill (window {window}, gated heads)", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t, byt(prompt), 4.0 * kw * H * hd, MFMA_BF16)
+            t = timed_k(lambda: hops.attn_tiles(q, hd ** -0.5, ngeom, window, sink0, vf, pos, seq, bt, t0, tn, kc, vc, H, hd))
+            add("nufalorn", f"attn_tiles prefill (block mask {window}, sink, turned values)", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t, byt(prompt), 4.0 * kb * H * hd, MFMA_BF16)
+            t = timed_k(lambda: hops.attn_tiles(q, hd ** -0.5, geom, 0, None, None, pos, seq, bt, t0, tn, kc, vc, H, hd, softcap=30.0, out_gate=og))
+            add("nepudra", "attn_tiles prefill (causal, capped scores, gated heads)", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t, byt(prompt), 4.0 * kc_ * H * hd, MFMA_BF16)
+            t = timed_k(lambda: hops.attn_tiles(q, hd ** -0.5, ngeom, 0, sink0, vf, pos, seq, bt, t0, tn, kc, vc, H, hd))
+            add("nufalorn", "attn_tiles prefill (causal, sink, turned values)", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t, byt(prompt), 4.0 * kc_ * H * hd, MFMA_BF16)
+        else:
+            t = timed_k(lambda: hops.attn_rows(q, hd ** -0.5, geom, 0, None, None, pos, seq, bt, kc, vc, H, hd, window=window, out_gate=og))
+            add("nepudra", f"attn_rows decode (window {window}, gated heads)", f"T=1 H={H} G={G} hd={hd} ctx={prompt}", t, byt(window), 4.0 * kw * H * hd, MFMA_BF16)
+            t = timed_k(lambda: hops.attn_rows(q, hd ** -0.5, ngeom, window, sink0, vf, pos, seq, bt, kc, vc, H, hd))
+            add("nufalorn", f"attn_rows decode (block mask {window})", f"T=1 H={H} G={G} hd={hd} ctx={prompt}", t, byt(window), 4.0 * kb * H * hd, MFMA_BF16)
+            t = timed_k(lambda: hops.attn_rows(q, hd ** -0.5, geom, 0, None, None, pos, seq, bt, kc, vc, H, hd, softcap=30.0, out_gate=og))
+            add("nepudra", "attn_rows decode (causal, capped scores, gated heads)", f"T=1 H={H} G={G} hd={hd} ctx={prompt}", t, byt(prompt), 4.0 * kc_ * H * hd, MFMA_BF16)
+            t = timed_k(lambda: hops.attn_rows(q, hd ** -0.5, ngeom, 0, sink0, vf, pos, seq, bt, kc, vc, H, hd))
+            add("nufalorn", "attn_rows decode (causal)", f"T=1 H={H} G={G} hd={hd} ctx={prompt}", t, byt(prompt), 4.0 * kc_ * H * hd, MFMA_BF16)
+    # before the scores: head norms + scaled turn + page write, and temperature + page write, against turn + value norm + page write
+    freq = torch.ones(hd // 2, device=dev) * 1e-3
+    qn, kn = bf(hd), bf(hd)
+    for T_ in (prompt, 8):
+        pos, seq = torch.arange(T_, dtype=torch.int32, device=dev), torch.zeros(T_, dtype=torch.int32, device=dev)
+        qkv = f32(T_, (H + 2 * G) * hd + H)
+        nb = T_ * ((H + 2 * G) * hd * 4 + H * hd * 4 + 2 * G * hd * 2)
+        t = timed_k(lambda: hops.attn_prep(qkv, H * hd, (H + G) * hd, geom, freq, None, False, 1e-6, pos, seq, bt, kc, vc, q_norm=qn, k_norm=kn, mag=1.2))
+        add("nepudra", "attn_prep (head norms, scaled turn)", f"T={T_} H={H} G={G}", t, nb, 0, VALU_F32)
+        g0 = hops.attn_geometry(H, G, hd, hd, 0, 0, 0, page, nblk, nblk)
+        t = timed_k(lambda: hops.attn_prep(qkv, H * hd, (H + G) * hd, g0, None, None, False, 1e-6, pos, seq, bt, kc, vc, q_temp=(0.2, 128)))
+        add("nepudra", "attn_prep (query temperature)", f"T={T_} H={H} G={G}", t, nb, 0, VALU_F32)
+        t = timed_k(lambda: hops.attn_prep(qkv, H * hd, (H + G) * hd, ngeom, freq, vf, True, 1e-5, pos, seq, bt, kc, vc))
+        add("nufalorn", "attn_prep (turn, value norm + turn)", f"T={T_} H={H} G={G}", t, nb, 0, VALU_F32)
+    # recurrence: the delta rule (width / 64 heads of 64 x 64) against the gated-linear-attention scan (heads of 64 x 128), and their head norms
+    Hd, d = W // 64, 64
+    for T_, name in ((prompt, "prefill"), (8, "decode b=8")):
+        nseq = 1 if T_ > 8 else 8
+        rs = torch.arange(0, T_ + 1, T_ // nseq, dtype=torch.int32, device=dev)
+        slot, fp = torch.arange(nseq, dtype=torch.int32, device=dev), torch.ones(nseq, dtype=torch.int32, device=dev)
+        proj, z = f32(T_, 5 * Hd * d), f32(T_, Hd * d)
+        state = torch.zeros(nseq, Hd, d, d, device=dev)
+        t = timed_k(lambda: hops.delta_scan(proj, 0, Hd * d, 2 * Hd * d, 3 * Hd * d, z, 0.6, 1e-6, Hd, d, d, rs, slot, fp, state))
+        add("nepudra", f"delta scan {name}", f"T={T_} H={Hd} dim={d} vdim={d}", t, T_ * 6 * Hd * d * 4 + 2 * nseq * Hd * d * d * 4, 8.0 * T_ * Hd * d * d, VALU_F32)
+        dg = hd // 2
+        pg, zg = f32(T_, 2 * H * dg + 2 * H * hd), f32(T_, H * dg)
+        sg = torch.zeros(nseq, H, dg, hd, device=dev)
+        t = timed_k(lambda: hops.scan(hops.SCAN_GLA, pg, 0, H * dg, 2 * H * dg, zg, None, None, 16.0, dg ** -0.5, H, dg, hd, rs, slot, fp, sg, torch.bfloat16))
+        add("nufalorn", f"scan GLA {name}", f"T={T_} H={H} dim={dg} vdim={hd}", t, T_ * (3 * H * dg + 2 * H * hd) * 4 + 2 * nseq * H * dg * hd * 4, 4.0 * T_ * H * dg * hd, VALU_F32)
+        o, wn = f32(T_, Hd * d), bf(Hd * d)
+        t = timed_k(lambda: hops.head_norm(o, Hd, d, wn, 1e-6, proj, 4 * Hd * d, gate_act="sigmoid"))
+        add("nepudra", f"head norm (weight per channel, sigmoid gate) {name}", f"T={T_} H={Hd} vdim={d}", t, T_ * Hd * d * 10, 0, VALU_F32)
+        og_, wg = f32(T_, H * hd), bf(hd)
+        t = timed_k(lambda: hops.head_norm(og_, H, hd, wg, 1e-5, pg, 2 * H * dg + H * hd))
+        add("nufalorn", f"head norm (shared weight, silu gate) {name}", f"T={T_} H={H} vdim={hd}", t, T_ * H * hd * 10, 0, VALU_F32)
+    # the layer's end: residual update + average over the stack's depth + norm, against residual update + two norms; embedding rows
+    for T_ in (prompt, 8):
+        x, a, b = f32(T_, W), f32(T_, W), f32(T_, W)
+        w1, w2 = bf(W), bf(W)
+        for n in (1, L // 2, L):
+            stack, coef = f32(n + 1, T_, W), f32(n + 1)
+            t = timed_k(lambda: hops.depth_mix_norm(x, a, stack, n, coef, w1, 1e-6))
+            add("nepudra", f"residual + depth average over {n + 1} + norm", f"M={T_} W={W}", t, stream_bytes(T_, W, n + 4, 1), 2.0 * T_ * W * (n + 1), VALU_F32)
+        t = timed_k(lambda: hops.residual_norm(x, a, None, 1.0, w1, None, 1e-6))
+        add("nepudra", "residual + norm (between the sublayers)", f"M={T_} W={W}", t, stream_bytes(T_, W, 3, 1), 0, VALU_F32)
+        t = timed_k(lambda: hops.residual_norm(x, a, b, 0.3, w1, w2, 1e-5, weight_offset=1.0))
+        add("nufalorn", "residual + 2 norms (fp32 stream)", f"M={T_} W={W}", t, stream_bytes(T_, W, 4, 2), 0, VALU_F32)
+        ids, prev = torch.randint(0, s["vocab"], (T_,), device=dev, dtype=torch.int32), torch.randint(0, s["vocab"], (T_,), device=dev, dtype=torch.int32)
+        table, bg, copy = bf(s["vocab"], W), bf(65522, W), f32(T_, W)
+        t = timed_k(lambda: hops.embed(ids, table, prev=prev, bigram=bg, mul_prev=8191, mul_cur=131, copy=copy))
+        add("nepudra", "embedding + bigram row (two copies)", f"M={T_} W={W}", t, T_ * W * (2 * 2 + 2 * 4), 0, VALU_F32)
+        t = timed_k(lambda: hops.embed(ids, table))
+        add("nufalorn", "embedding", f"M={T_} W={W}", t, T_ * W * (2 + 4), 0, VALU_F32)
+    # linears: the one input linear of a delta layer (r | k | v | a | g, biased, fp32 out), the gelu-gated MLP against the relu-gated one
+    for M_ in (prompt, 8, 1):
+        x = bf(M_, W)
+        w5, b5 = bf(5 * W, W), bf(5 * W)
+        t = timed_k(lambda: hops.dense_linear(x, w5, b5, out_dtype=torch.float32))
+        add("nepudra", "dense_linear r|k|v|a|g (bias, fp32 out)", f"M={M_} N={5 * W} K={W}", t, 5 * W * W * 2 + M_ * (W * 2 + 5 * W * 4), 2.0 * M_ * 5 * W * W, MFMA_BF16)
+        wq = bf((H + 2 * G) * hd, W)
+        t = timed_k(lambda: hops.dense_linear(x, wq, out_dtype=torch.float32))
+        add("nufalorn", "dense_linear q|k|v (fp32 out)", f"M={M_} N={(H + 2 * G) * hd} K={W}", t, (H + 2 * G) * hd * W * 2 + M_ * (W * 2 + (H + 2 * G) * hd * 4),
+            2.0 * M_ * (H + 2 * G) * hd * W, MFMA_BF16)
+        wgu = hops.group_gate_up(bf(ff, W), bf(ff, W))
+        for fam, act in (("nepudra", hops.ACT_GELU_TANH), ("nufalorn", hops.ACT_RELU)):
+            t = timed_k(lambda: hops.dense_linear(x, wgu, gated=True, act=act))
+            add(fam, "dense_linear gated (%s)" % ("gelu" if fam == "nepudra" else "relu"), f"M={M_} N={2 * ff} K={W}", t, 2 * ff * W * 2 + M_ * (W + ff) * 2,
+                2.0 * M_ * 2 * ff * W, MFMA_BF16)
+    return rows
+
+
 def stream_bytes(T_, W, f32_streams, bf16_streams):
     return T_ * W * (4 * f32_streams + 2 * bf16_streams)
 
 
-def run_pokepel(args, dev, sizes):
+def run_pokepel(args, dev, sizes, member="pokepel"):
     prompt, batch, steps = args.hybrid_prompt, args.hybrid_batch, args.steps
     out = {}
     for name in sizes:
         s = SIZES[name]
         log(f"[hybrid bench] {name}: {s}")
         rec = {"config": s, "prompt": prompt, "batch": batch}
-        for design in ("pokepel", "nufalorn"):
+        for design in (member, "nufalorn"):
             rec[design], model, eng = bench_hybrid_engine(s, dev, prompt, batch, steps, design)
             del model, eng
             torch.cuda.empty_cache()
             log(f"[hybrid bench] {name} {design}: {rec[design]}")
-        rec["kernels"] = kernel_table_pokepel(s, dev, prompt)
+        rec["kernels"] = (kernel_table_pokepel if member == "pokepel" else kernel_table_nepudra)(s, dev, prompt)
         for r in rec["kernels"]:
-            log(f"    {r['family']:8s} {r['kernel']:44s} {r['shape']:48s} {r['us']:10.1f} us  roofline {r['roofline_us']:9.2f} us  x{r['x_roofline']}")
+            log(f"    {r['family']:8s} {r['kernel']:64s} {r['shape']:48s} {r['us']:10.1f} us  roofline {r['roofline_us']:9.2f} us  x{r['x_roofline']}")
         out[name] = rec
-    print(json.dumps({"hybrid_bench": out, "design": "pokepel", "dtype": "bf16", "data": "synthetic (random weights and tokens)"}))
+    print(json.dumps({"hybrid_bench": out, "design": member, "dtype": "bf16", "data": "synthetic (random weights and tokens)"}))
     return 0
 
 
@@ -475,8 +666,8 @@ def run(args):
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     sizes = [x for x in (args.hybrid_sizes.split(",") if args.hybrid_sizes else SIZES)]
-    if getattr(args, "hybrid_design", "nufalorn") == "pokepel":
-        return run_pokepel(args, dev, sizes)
+    if getattr(args, "hybrid_design", "nufalorn") in ("pokepel", "nepudra"):
+        return run_pokepel(args, dev, sizes, args.hybrid_design)
     prompt, batch, steps = args.hybrid_prompt, args.hybrid_batch, args.steps
     out = {}
     for name in sizes:

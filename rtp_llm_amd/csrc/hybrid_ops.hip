@@ -888,9 +888,9 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
 // ------------------------------------------------------------------------------------------------ generalized delta rule
 // S_t = diag(w_t) S_(t-1) - (a_t * u_t)(u_t^T S_(t-1)) + k_t v_t^T, o_t = S_t^T r_t per head, S [dim (key channel), vdim] in an fp32 slot; both the
 // decayed and the removed term read the old state.  w = exp(-decay_mult * sigmoid(z)), a = sigmoid(removal pre-activation), u = k / sqrt(|k|^2 +
-// unit_eps) over the head's key channels: all in fp32.  A quad of lanes owns one value column, each lane RD of its key rows; a wave owns 16 columns
-// and a block of four waves 64.  Per token the only exchange is the quad sum of u^T S (and of the output), two DPP steps each; the gates of `tok`
-// tokens are computed once into LDS by the whole block.  The walk over a sequence's tokens is the same arithmetic however the tokens were cut into steps.
+// unit_eps) over the head's key channels: all in fp32.  A group of neighbouring lanes owns one value column, each lane some of its key rows.  Per
+// token the only exchange is the group's sum of u^T S (and of the output) by DPP steps; the gates of a pass of tokens are computed once into LDS by
+// the whole block.  The walk over a sequence's tokens is the same arithmetic however the tokens were cut into steps.
 struct DeltaParams {
     const float* proj; int ld; int ro, ko, vo, ao;   // fp32 projections [rows, ld]: r, k, v heads and the removal pre-activation at these columns
     const float* z; int ldz;                          // decay pre-activation [rows, H * dim]
@@ -899,29 +899,27 @@ struct DeltaParams {
     const int32_t* row_start; const int32_t* slot; const int32_t* first_pos;
     float* state;                                     // [slots, H, dim, vdim]
     float* out;                                       // [rows, H * vdim]
-    int tok;
+    int reserved;
 };
 
-__device__ __forceinline__ float hy_quad_sum(float v) {
-    v += hy_dpp<0xB1>(v);      // quad_perm [1,0,3,2]
+template <int LPC> __device__ __forceinline__ float hy_lanes_sum(float v);
+template <> __device__ __forceinline__ float hy_lanes_sum<4>(float v) {
+    v += hy_dpp<0xB1>(v);        // quad_perm [1,0,3,2]
     return v + hy_dpp<0x4E>(v);  // quad_perm [2,3,0,1]
 }
+template <> __device__ __forceinline__ float hy_lanes_sum<16>(float v) { return hy_sum16(v); }
 
-template <int RD>
+// LPC lanes (4 or 16, neighbours inside a DPP row) own one value column, each RD key rows of it (dim <= LPC * RD); a wave owns 64 / LPC columns and a
+// block of four waves CW = 256 / LPC.  Sixteen lanes per column keep the per-token chain short (RD multiply-adds, four DPP steps), which is what a
+// single sequence's walk is bound by; TOK tokens are staged per pass, and the raw projections of the next pass are fetched during the walk.
+template <int RD, int LPC>
 __global__ __launch_bounds__(256) void hy_delta_kernel(DeltaParams p) {
-    extern __shared__ __attribute__((aligned(16))) float hy_dl[];
-    constexpr int dpad = 4 * RD;
-    const int TOK = p.tok;
-    float* w_s = hy_dl;                          // [TOK][dpad] each
-    float* b_s = w_s + TOK * dpad;
-    float* u_s = b_s + TOK * dpad;
-    float* k_s = u_s + TOK * dpad;
-    float* r_s = k_s + TOK * dpad;
-    float* v_s = r_s + TOK * dpad;               // [TOK][64]
-    float* o_s = v_s + TOK * 64;                 // [TOK][64]
-    float* inv_s = o_s + TOK * 64;               // [TOK]
-    const int sq = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * 64;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rg = lane & 3, col = wave * 16 + (lane >> 2);
+    constexpr int dpad = LPC * RD, CW = 256 / LPC, TOK = dpad <= 128 ? 16 : 8;
+    constexpr int EL = (TOK * dpad + 255) / 256, VE = (TOK * CW + 255) / 256;
+    __shared__ __attribute__((aligned(16))) float w_s[TOK * dpad], b_s[TOK * dpad], u_s[TOK * dpad], k_s[TOK * dpad], r_s[TOK * dpad];
+    __shared__ float v_s[TOK * CW], o_s[TOK * CW], inv_s[TOK];
+    const int sq = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * CW;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rg = lane % LPC, col = wave * (64 / LPC) + lane / LPC;
     const int r0 = p.row_start[sq], r1 = p.row_start[sq + 1];
     const bool vok = v0 + col < p.vdim;
     float* st = p.state + (((size_t)p.slot[sq] * p.H + h) * p.dim) * p.vdim + v0 + col;
@@ -932,68 +930,108 @@ __global__ __launch_bounds__(256) void hy_delta_kernel(DeltaParams p) {
         const int d = rg * RD + j;
         S[j] = (!fresh && vok && d < p.dim) ? st[(size_t)d * p.vdim] : 0.f;
     }
-    for (int t0 = r0; t0 < r1; t0 += TOK) {
+    float fr[EL], fk[EL], fa[EL], fz[EL], fv[VE];
+    auto fetch = [&](int t0) {
         const int nt = min(TOK, r1 - t0);
-        for (int i = tid; i < nt * dpad; i += 256) {
-            const int t = i / dpad, d = i % dpad;
-            float rv = 0.f, kv = 0.f, wv = 1.f, av = 0.f;
-            if (d < p.dim) {
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+            const int i = tid + e * 256, t = i / dpad, d = i % dpad;
+            fr[e] = fk[e] = fa[e] = fz[e] = 0.f;
+            if (i < nt * dpad && d < p.dim) {
                 const float* row = p.proj + (size_t)(t0 + t) * p.ld;
                 const int hd = h * p.dim + d;
-                rv = row[p.ro + hd]; kv = row[p.ko + hd];
-                av = hy_sigmoid(row[p.ao + hd]);
-                wv = expf(-p.decay_mult * hy_sigmoid(p.z[(size_t)(t0 + t) * p.ldz + hd]));
+                fr[e] = row[p.ro + hd]; fk[e] = row[p.ko + hd]; fa[e] = row[p.ao + hd];
+                fz[e] = p.z[(size_t)(t0 + t) * p.ldz + hd];
             }
-            r_s[i] = rv; k_s[i] = kv; w_s[i] = wv; b_s[i] = av;
         }
-        for (int i = tid; i < nt * 64; i += 256)
-            v_s[i] = (v0 + (i & 63) < p.vdim) ? p.proj[(size_t)(t0 + (i >> 6)) * p.ld + p.vo + h * p.vdim + v0 + (i & 63)] : 0.f;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+            const int i = tid + e * 256, cc = i % CW;
+            fv[e] = (i < nt * CW && v0 + cc < p.vdim) ? p.proj[(size_t)(t0 + i / CW) * p.ld + p.vo + h * p.vdim + v0 + cc] : 0.f;
+        }
+    };
+    if (r0 < r1) fetch(r0);
+    for (int t0 = r0; t0 < r1; t0 += TOK) {
+        const int nt = min(TOK, r1 - t0);
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+            const int i = tid + e * 256, d = i % dpad;
+            if (i >= nt * dpad) continue;
+            const bool in = d < p.dim;                  // rows beyond the key size: zero keys, no removal, state stays zero
+            r_s[i] = fr[e]; k_s[i] = fk[e];
+            b_s[i] = in ? hy_sigmoid(fa[e]) : 0.f;
+            w_s[i] = in ? expf(-p.decay_mult * hy_sigmoid(fz[e])) : 1.f;
+        }
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+            const int i = tid + e * 256;
+            if (i < nt * CW) v_s[i] = fv[e];
+        }
         __syncthreads();
-        for (int t = wave; t < nt; t += 4) {         // |k|^2 of a token's head: one wave
+        {                                             // |k|^2 of a token's head: sixteen neighbouring lanes per token (TOK <= 16 tokens, 256 threads)
+            const int t = tid >> 4, l = tid & 15;
             float ss = 0.f;
-            for (int d = lane; d < p.dim; d += 64) ss = __builtin_fmaf(k_s[t * dpad + d], k_s[t * dpad + d], ss);
-            ss = hy_wave_sum(ss);
-            if (lane == 0) inv_s[t] = 1.f / sqrtf(ss + p.unit_eps);
+            if (t < nt)
+                for (int d = l; d < dpad; d += 16) ss = __builtin_fmaf(k_s[t * dpad + d], k_s[t * dpad + d], ss);
+            ss = hy_sum16(ss);
+            if (t < nt && l == 0) inv_s[t] = 1.f / sqrtf(ss + p.unit_eps);
         }
         __syncthreads();
-        for (int i = tid; i < nt * dpad; i += 256) {
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+            const int i = tid + e * 256;
+            if (i >= nt * dpad) continue;
             const float u = k_s[i] * inv_s[i / dpad];
             u_s[i] = u; b_s[i] = b_s[i] * u;
         }
         __syncthreads();
-        for (int t = 0; t < nt; ++t) {
-            const float vt = v_s[t * 64 + col];
-            const f32x4* uu = (const f32x4*)(u_s + t * dpad + rg * RD);
-            const f32x4* ww = (const f32x4*)(w_s + t * dpad + rg * RD);
-            const f32x4* bb = (const f32x4*)(b_s + t * dpad + rg * RD);
-            const f32x4* kk = (const f32x4*)(k_s + t * dpad + rg * RD);
-            const f32x4* rr = (const f32x4*)(r_s + t * dpad + rg * RD);
+        if (t0 + TOK < r1) fetch(t0 + TOK);          // in flight during the walk
+        // the gates of token t + 1 are read from LDS while token t is worked on (two register sets, taken in turns)
+        struct Gates { f32x4 u[RD / 4], w[RD / 4], b[RD / 4], k[RD / 4], r[RD / 4]; float v; };
+        auto load = [&](int t, Gates& g) {
+            const int o = t * dpad + rg * RD;
+#pragma unroll
+            for (int j4 = 0; j4 < RD / 4; ++j4) {
+                g.u[j4] = *(const f32x4*)(u_s + o + j4 * 4); g.w[j4] = *(const f32x4*)(w_s + o + j4 * 4); g.b[j4] = *(const f32x4*)(b_s + o + j4 * 4);
+                g.k[j4] = *(const f32x4*)(k_s + o + j4 * 4); g.r[j4] = *(const f32x4*)(r_s + o + j4 * 4);
+            }
+            g.v = v_s[t * CW + col];
+        };
+        auto step = [&](int t, const Gates& g) {
             float sp[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j4 = 0; j4 < RD / 4; ++j4) {
-                const f32x4 u4 = uu[j4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) sp[e] = __builtin_fmaf(u4[e], S[j4 * 4 + e], sp[e]);
+                for (int e = 0; e < 4; ++e) sp[e] = __builtin_fmaf(g.u[j4][e], S[j4 * 4 + e], sp[e]);
             }
-            const float sb = hy_quad_sum((sp[0] + sp[1]) + (sp[2] + sp[3]));      // (u^T S_old)[column]
+            const float sb = hy_lanes_sum<LPC>((sp[0] + sp[1]) + (sp[2] + sp[3]));      // (u^T S_old)[column]
             float op[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j4 = 0; j4 < RD / 4; ++j4) {
-                const f32x4 w4 = ww[j4], b4 = bb[j4], k4 = kk[j4], r4 = rr[j4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int j = j4 * 4 + e;
-                    S[j] = __builtin_fmaf(w4[e], S[j], __builtin_fmaf(-b4[e], sb, k4[e] * vt));
-                    op[e] = __builtin_fmaf(r4[e], S[j], op[e]);
+                    S[j] = __builtin_fmaf(g.w[j4][e], S[j], __builtin_fmaf(-g.b[j4][e], sb, g.k[j4][e] * g.v));
+                    op[e] = __builtin_fmaf(g.r[j4][e], S[j], op[e]);
                 }
             }
-            const float o = hy_quad_sum((op[0] + op[1]) + (op[2] + op[3]));
-            if (rg == 0) o_s[t * 64 + col] = o;
+            const float o = hy_lanes_sum<LPC>((op[0] + op[1]) + (op[2] + op[3]));
+            if (rg == 0) o_s[t * CW + col] = o;
+        };
+        Gates ga, gb;
+        load(0, ga);
+        for (int t = 0; t < nt; t += 2) {
+            load(min(t + 1, nt - 1), gb);
+            step(t, ga);
+            if (t + 1 < nt) {
+                load(min(t + 2, nt - 1), ga);
+                step(t + 1, gb);
+            }
         }
         __syncthreads();
-        for (int i = tid; i < nt * 64; i += 256) {
-            const int cc = i & 63;
-            if (v0 + cc < p.vdim) p.out[(size_t)(t0 + (i >> 6)) * p.H * p.vdim + h * p.vdim + v0 + cc] = o_s[i];
+        for (int i = tid; i < nt * CW; i += 256) {
+            const int cc = i % CW;
+            if (v0 + cc < p.vdim) p.out[(size_t)(t0 + i / CW) * p.H * p.vdim + h * p.vdim + v0 + cc] = o_s[i];
         }
     }
     if (vok) {
@@ -1504,19 +1542,16 @@ extern "C" int mi355_hy_delta_scan(const float* proj, int32_t ld, int32_t ro, in
     MI355_CHECK_ARG(proj && z && row_start && slot && first_pos && state && out && nseq > 0 && H > 0 && dim > 0 && vdim > 0, "hy_delta_scan: bad argument");
     MI355_CHECK_ARG(dim <= 256, "hy_delta_scan: key size %d > 256", dim);
     MI355_CHECK_ARG(ld >= H * dim && ldz >= H * dim && unit_eps >= 0.f, "hy_delta_scan: ld=%d ldz=%d", ld, ldz);
-    const int RD = dim <= 16 ? 4 : dim <= 32 ? 8 : dim <= 64 ? 16 : dim <= 128 ? 32 : 64;
-    int tok = 16;
-    auto lds_of = [&](int t) { return (size_t)(5 * t * 4 * RD + 2 * t * 64 + t) * 4; };
-    while (tok > 1 && lds_of(tok) > 60 * 1024) tok >>= 1;
-    DeltaParams p{proj, ld, ro, ko, vo, ao, z, ldz, decay_mult, unit_eps, H, dim, vdim, row_start, slot, first_pos, state, out, tok};
-    const dim3 grid(nseq, H, (vdim + 63) / 64);
-    const size_t lds = lds_of(tok);
+    DeltaParams p{proj, ld, ro, ko, vo, ao, z, ldz, decay_mult, unit_eps, H, dim, vdim, row_start, slot, first_pos, state, out, 0};
     hipStream_t st = (hipStream_t)stream;
-    if (RD == 4)       hipLaunchKernelGGL(hy_delta_kernel<4>, grid, dim3(256), lds, st, p);
-    else if (RD == 8)  hipLaunchKernelGGL(hy_delta_kernel<8>, grid, dim3(256), lds, st, p);
-    else if (RD == 16) hipLaunchKernelGGL(hy_delta_kernel<16>, grid, dim3(256), lds, st, p);
-    else if (RD == 32) hipLaunchKernelGGL(hy_delta_kernel<32>, grid, dim3(256), lds, st, p);
-    else               hipLaunchKernelGGL(hy_delta_kernel<64>, grid, dim3(256), lds, st, p);
+    // sixteen lanes per value column (16 columns per block) for heads of more than 32 key channels, four (64 columns per block) below
+    const dim3 g16(nseq, H, (vdim + 15) / 16), g4(nseq, H, (vdim + 63) / 64);
+    if (dim <= 16)       hipLaunchKernelGGL((hy_delta_kernel<4, 4>), g4, dim3(256), 0, st, p);
+    else if (dim <= 32)  hipLaunchKernelGGL((hy_delta_kernel<8, 4>), g4, dim3(256), 0, st, p);
+    else if (dim <= 64)  hipLaunchKernelGGL((hy_delta_kernel<4, 16>), g16, dim3(256), 0, st, p);
+    else if (dim <= 128) hipLaunchKernelGGL((hy_delta_kernel<8, 16>), g16, dim3(256), 0, st, p);
+    else if (dim <= 192) hipLaunchKernelGGL((hy_delta_kernel<12, 16>), g16, dim3(256), 0, st, p);
+    else                 hipLaunchKernelGGL((hy_delta_kernel<16, 16>), g16, dim3(256), 0, st, p);
     MI355_CHECK_LAUNCH("hy_delta_kernel");
     return MI355_OK;
 }
