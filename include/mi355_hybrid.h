@@ -12,11 +12,12 @@ extern "C" {
 #endif
 
 /* ------------------------------------------------------------------------------------------------------------------------------
- * libmi355_hybrid.so: dense linears on [out, in] weights and the kernels of the hybrid decoder family (parallel-residual layers
- * over an fp32 stream; token mixers: paged chunk-masked attention with a softmax sink and position-rotated values, and gated
+ * libmi355_hybrid.so: dense linears on [out, in] weights and the kernels of the hybrid decoder family (parallel-residual or sequential
+ * layers over an fp32 stream; token mixers: paged chunk-masked attention with a softmax sink and position-rotated values, and gated
  * linear recurrences with fp32 state slots; low-rank latent attention over one cached row per token, fixed-decay retention, PolyNorm,
- * sigmoid-gated branches, group-limited mixtures of experts over grouped linears; sliding-window and score-capped attention with per-head output gates,
- * normed queries and keys, a generalized delta-rule recurrence, hashed bigram embedding rows, a weighted average over the depth of the stack).  act_dtype is MI355_ACT_BF16 or MI355_ACT_F32.  Sources: csrc/gemm_dense.hip,
+ * sigmoid-gated branches, group-limited mixtures of experts over grouped linears; sliding-window and score-capped attention with
+ * per-head output gates and normed queries and keys, a generalized delta-rule recurrence, hashed bigram embedding rows, a weighted
+ * average over the depth of the stack).  act_dtype is MI355_ACT_BF16 or MI355_ACT_F32.  Sources: csrc/gemm_dense.hip,
  * csrc/hybrid_ops.hip; the argument conventions are documented at the definitions. */
 int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y, int32_t ldy,
                        int32_t out_f32, int32_t gated, int32_t act, float softcap, int32_t act_dtype, mi355_stream_t stream);

@@ -3,7 +3,11 @@
 // denominator, optionally unit-normed values that are rotated by their position and turned back at the query's position; or low-rank latent
 // attention over one cached row per token that serves as key and, with its leading channels, as value) or a linear recurrence
 // S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with its state in fp32 slots (HGRN2, gated-linear-attention and fixed-decay retention
-// parametrisations of a, k, q); feed-forward helpers: PolyNorm, and routing / sorting / weighted sum of a mixture of experts.
+// parametrisations of a, k, q; or the generalized delta rule S_t = diag(w_t) S_(t-1) - (a_t * u_t)(u_t^T S_(t-1)) + k_t v_t^T); feed-forward
+// helpers: PolyNorm, and routing / sorting / weighted sum of a mixture of experts.  Options of the attention kernels: sliding window, tanh
+// cap on the scores, per-head sigmoid gate on the output, normed queries and keys, scaled rotary magnitude, a query temperature.  For members
+// whose sublayers follow each other: the layer's end as residual update + weighted average over the results of all earlier layers + norm,
+// and a hashed bigram row beside the token embedding.
 //
 // One ragged batch of rows serves prefill portions and decode tokens alike: every row carries its position and the index of its
 // sequence; a sequence carries its block-table row, its state slot and the range of its rows.  What the model states as 32-bit is fp32

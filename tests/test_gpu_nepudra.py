@@ -492,6 +492,22 @@ def test_long_decoding():
     close(out, ref[10:], 5e-4)
 
 
+def test_contexts_beyond_a_thousand_tokens_split_decode_rows():
+    """Past 1024 cached tokens a decode row's keys are dealt over several blocks and merged by a second launch: cap, window start and head gate
+    must survive that path (causal layer, and a window wide enough to be split as well)."""
+    cfg = U.make_config([U.capped_layer(heads=2, kv_heads=1, softcap=6.0), U.window_layer(heads=2, kv_heads=1, window=1100, scaling=U.YARN)], vocab=50, width=32)
+    w = U.make_weights(cfg, seed=41)
+    t = toks(1180, 50, 42)
+    ref = U.oracle_logits(cfg, w, t)
+    eng = engine(cfg, w, max_tokens=1280)
+    close(eng.run_step([("d", t[:1140], [0, 700, 1139])]), ref[[0, 700, 1139]], 5e-4)
+    out = torch.cat([eng.run_step([("d", [tk], [0])]) for tk in t[1140:]])
+    close(out, ref[1140:], 5e-4)
+    eng = engine(cfg, w, torch.bfloat16, max_tokens=1280)
+    eng.run_step([("d", t[:1140], [])])
+    bf16_close(torch.cat([eng.run_step([("d", [tk], [0])]) for tk in t[1140:]]), ref[1140:])
+
+
 # ------------------------------------------------------------------------------------------------ generation
 def _oracle_greedy(cfg, w, prompt, n):
     seq, margins = list(prompt), []
