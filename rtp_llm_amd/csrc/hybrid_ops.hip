@@ -903,7 +903,6 @@ struct DeltaParams {
     const int32_t* row_start; const int32_t* slot; const int32_t* first_pos;
     float* state;                                     // [slots, H, dim, vdim]
     float* out;                                       // [rows, H * vdim]
-    int reserved;
 };
 
 template <int LPC> __device__ __forceinline__ float hy_lanes_sum(float v);
@@ -1546,7 +1545,7 @@ extern "C" int mi355_hy_delta_scan(const float* proj, int32_t ld, int32_t ro, in
     MI355_CHECK_ARG(proj && z && row_start && slot && first_pos && state && out && nseq > 0 && H > 0 && dim > 0 && vdim > 0, "hy_delta_scan: bad argument");
     MI355_CHECK_ARG(dim <= 256, "hy_delta_scan: key size %d > 256", dim);
     MI355_CHECK_ARG(ld >= H * dim && ldz >= H * dim && unit_eps >= 0.f, "hy_delta_scan: ld=%d ldz=%d", ld, ldz);
-    DeltaParams p{proj, ld, ro, ko, vo, ao, z, ldz, decay_mult, unit_eps, H, dim, vdim, row_start, slot, first_pos, state, out, 0};
+    DeltaParams p{proj, ld, ro, ko, vo, ao, z, ldz, decay_mult, unit_eps, H, dim, vdim, row_start, slot, first_pos, state, out};
     hipStream_t st = (hipStream_t)stream;
     // sixteen lanes per value column (16 columns per block) for heads of more than 32 key channels, four (64 columns per block) below
     const dim3 g16(nseq, H, (vdim + 15) / 16), g4(nseq, H, (vdim + 63) / 64);

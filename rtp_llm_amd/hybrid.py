@@ -158,13 +158,13 @@ def nepudra_from_json(cfg: dict) -> HybridConfig:
             spec, kind = DeltaRuleSpec(heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx["dim"])), "delta_rule"
         elif kind == "attention":
             qt = mx.get("q_temp")
-            spec = AttentionSpec(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]), vdim=int(mx["vdim"]),
-                                 scale=float(mx["scale"]), kv_from=src, softcap=float(mx.get("softcap") or 0.0),
+            spec = AttentionSpec(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]), vdim=int(mx.get("vdim", mx["dim"])),
+                                 scale=float(mx.get("scale", int(mx["dim"]) ** -0.5)), kv_from=src, softcap=float(mx.get("softcap") or 0.0),
                                  q_temp=(float(qt["coef"]), int(qt["every"])) if qt else None, bias=True, out_bias=True, out_gate=True)
         elif kind == "attention_2":
             mask = mx.get("mask") or {}
-            spec = AttentionSpec(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]), vdim=int(mx["vdim"]),
-                                 scale=float(mx["scale"]), rot=RotarySpec.from_json(mx.get("rot"), "halves"), kv_from=src,
+            spec = AttentionSpec(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]), vdim=int(mx.get("vdim", mx["dim"])),
+                                 scale=float(mx.get("scale", int(mx["dim"]) ** -0.5)), rot=RotarySpec.from_json(mx.get("rot"), "halves"), kv_from=src,
                                  window=int(mask.get("size", 0) or 0), qk_norm=True, bias=True, out_gate=True)
             kind = "attention"
         else:
@@ -273,7 +273,7 @@ class HybridModel:
                 gate_w = torch.cat([mixer.w_in, zrow, gate_w], 0).contiguous()
                 mixer.w_in = None                      # lives on as the leading rows of the shared weight
             self.layers.append((L, mixer, mlp, norm_w(p + "norm1"), n2, gate_w, gate_b))
-        self.has_state = any(L.kind not in ("attention", "latent_attention") for L in cfg.layers) or cfg.bigram is not None
+        self.has_state = any(L.kind not in ("attention", "latent_attention") for L in cfg.layers)
 
     # ---- what an engine has to allocate
     def cache_layout(self):
