@@ -87,6 +87,31 @@ int mi355_hy_delta_scan(const float* proj, int32_t ld, int32_t ro, int32_t ko, i
                         float decay_mult, float unit_eps, int32_t H, int32_t dim, int32_t vdim, const int32_t* row_start, const int32_t* slot,
                         const int32_t* first_pos, int32_t nseq, float* state, float* out, mi355_stream_t stream);
 
+
+/* Further extended forms: an activation with a parameter (act 5: clamped gated form g' sigmoid(1.702 g') (u' + 1)), routers that score by sigmoids, rank
+ * groups by their two best experts and scale the weights, a query / key norm over all heads at once, an embedding with a multiplier, and the end of a
+ * sublayer whose output is normed before it joins the stream (layer norm or RMS norm), also as the last norm on gathered rows. */
+int mi355_dense_linear_ex(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y, int32_t ldy,
+                          int32_t out_f32, int32_t gated, int32_t act, float act_param, float softcap, int32_t act_dtype, mi355_stream_t stream);
+int mi355_dense_grouped_ex(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y, int32_t ldy,
+                           int32_t out_f32, int32_t gated, int32_t act, float act_param, int32_t act_dtype, int32_t G, int64_t xs, int64_t ys,
+                           const int32_t* offs, const int32_t* gather, const int32_t* tiles, int32_t max_tiles, const float* egate, int32_t ldg,
+                           int32_t goff, mi355_stream_t stream);
+int mi355_hy_moe_route_ex(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
+                          int32_t score_sigmoid, int32_t group_top, float wscale, mi355_stream_t stream);
+int mi355_hy_moe_route_align_ex(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
+                                int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles, int32_t score_sigmoid, int32_t group_top,
+                                float wscale, mi355_stream_t stream);
+int mi355_hy_attn_prep_ex2(float* qkv, int32_t ld, int32_t koff, int32_t voff, const int32_t* geom, const float* kfreq, const float* vfreq,
+                           int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
+                           void* kcache, void* vcache, const void* qnorm, const void* knorm, int32_t norm_whole, float mag, float qt_coef,
+                           int32_t qt_every, int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_embed_scaled(const int32_t* ids, int32_t rows, const void* table, int32_t W, int32_t vocab, float scale, float* out, void* outh,
+                          int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_branch_norm(float* x, const float* a, float ca, const float* b, float cb, const float* sh, const float* sg, int32_t ldsg,
+                         const float* moe_y, const int32_t* moe_place, const float* moe_wts, int32_t moe_top, const int32_t* self_rows, int32_t n,
+                         int32_t W, const void* w, int32_t center, float eps, void* h, int32_t act_dtype, mi355_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

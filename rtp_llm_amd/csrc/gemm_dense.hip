@@ -9,7 +9,8 @@
 //   * row kernel (M = 1; fp32 up to M = 16): a wave per output column streams its weight row once, 16-byte loads, wave reduction at the end.
 //   * grouped forms of the tile kernels (per-head weights over column slices, or rows sorted by expert with a gather and a tile list) and
 //     of the row kernel (the few rows of a decode step, each with its own expert's weight): mi355_dense_grouped.
-// Epilogues: bias, gated activation act(gate) * up (weight rows grouped [32 gate | 32 up], so one lane holds both), tanh soft cap.
+// Epilogues: bias, gated activation act(gate) * up (weight rows grouped [32 gate | 32 up], so one lane holds both; also the clamped form
+// min(g, L) sigmoid(1.702 min(g, L)) (clamp(u, -L, L) + 1)), tanh soft cap.
 // Output is fp32 or the activation type.  A result row depends only on its own input row: the k order of the accumulation is fixed by
 // the kernel, never by M or by the row's place in the batch.
 #include "common.h"
@@ -17,13 +18,14 @@
 
 namespace {
 
-constexpr int DN_ACT_NONE = 0, DN_ACT_RELU = 1, DN_ACT_SILU = 2, DN_ACT_GELU_TANH = 3, DN_ACT_TANH = 4;
+constexpr int DN_ACT_NONE = 0, DN_ACT_RELU = 1, DN_ACT_SILU = 2, DN_ACT_GELU_TANH = 3, DN_ACT_TANH = 4, DN_ACT_SWIGLU_CLAMP = 5;
 
 struct DenseParams {
     const void* x; const void* w; const void* bias; void* y;
     int M, N, K, ldx, ldy;
     int gated;       // 0: N outputs; 1: rows of w are [32 gate | 32 up] groups, N / 2 outputs
     int act;         // DN_ACT_* applied to the gate
+    float act_param; // DN_ACT_SWIGLU_CLAMP: the limit of the gate (from above) and of the up value (both sides)
     int out_f32;
     float softcap;   // > 0: y = cap * tanh(y / cap)
     int vec;         // 16-byte loads allowed (alignment and K % 8 == 0 checked on the host)
@@ -60,6 +62,15 @@ __device__ __forceinline__ float dn_act(float g, int act) {
     if (act == DN_ACT_GELU_TANH) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
     if (act == DN_ACT_TANH) return tanhf(g);
     return g;
+}
+
+// act(gate) * up of a gated pair.  DN_ACT_SWIGLU_CLAMP: g' = min(g, L), u' = clamp(u, -L, L), g' sigmoid(1.702 g') (u' + 1).
+__device__ __forceinline__ float dn_gated(float g, float u, int act, float lim) {
+    if (act == DN_ACT_SWIGLU_CLAMP) {
+        g = fminf(g, lim); u = fminf(fmaxf(u, -lim), lim);
+        return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+    }
+    return dn_act(g, act) * u;
 }
 
 template <typename T> __device__ __forceinline__ float dn_ld(const T* p) { return (float)*p; }
@@ -157,7 +168,7 @@ __global__ __launch_bounds__(256) void dense_tile_bf16_kernel(DenseParams p) {
                     if (ng + 32 >= p.N) continue;
                     float g = acc[i][j][e], u = acc[i][j + 2][e];
                     if (Bi) { g += dn_ld(Bi + ng); u += dn_ld(Bi + ng + 32); }
-                    dn_store<bf16>(p, row, (int)gr.yo + (ng >> 6) * 32 + (ng & 31), dn_act(g, p.act) * u);
+                    dn_store<bf16>(p, row, (int)gr.yo + (ng >> 6) * 32 + (ng & 31), dn_gated(g, u, p.act, p.act_param));
                 }
             } else {
 #pragma unroll
@@ -237,7 +248,7 @@ __global__ __launch_bounds__(256) void dense_tile_f32_kernel(DenseParams p) {
                 if (n + 32 >= p.N) continue;
                 float g = acc[i][j], u = acc[i][j + 2];
                 if (Bi) { g += Bi[n]; u += Bi[n + 32]; }
-                dn_store<float>(p, row, (int)gr.yo + (n >> 6) * 32 + (n & 31), dn_act(g, p.act) * u);
+                dn_store<float>(p, row, (int)gr.yo + (n >> 6) * 32 + (n & 31), dn_gated(g, u, p.act, p.act_param));
             } else {
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
@@ -336,8 +347,7 @@ __global__ __launch_bounds__(256) void dense_rows_kernel(DenseParams p, int mbas
             if (lane != 0 || o >= nout) continue;
             const int n0 = GATED ? (o >> 5) * 64 + (o & 31) : o;
             if (p.bias) { g += dn_ld((const T*)p.bias + n0); if (GATED) u += dn_ld((const T*)p.bias + n0 + 32); }
-            g = dn_act(g, p.act);
-            dn_store<T>(p, mbase + m, o, GATED ? g * u : g);
+            dn_store<T>(p, mbase + m, o, GATED ? dn_gated(g, u, p.act, p.act_param) : dn_act(g, p.act));
         }
     }
 }
@@ -386,8 +396,7 @@ __global__ __launch_bounds__(256) void dense_rows_grouped_kernel(DenseParams p) 
         const float u = GATED ? dn_wave_sum(a1[c]) : 0.f;
         const int o = o0 + c;
         if (lane != 0 || o >= nout) continue;
-        gsum = dn_act(gsum, p.act);
-        dn_store<T>(p, r, (int)(p.ys * g) + o, GATED ? gsum * u : gsum);
+        dn_store<T>(p, r, (int)(p.ys * g) + o, GATED ? dn_gated(gsum, u, p.act, p.act_param) : dn_act(gsum, p.act));
     }
 }
 
@@ -457,8 +466,7 @@ __global__ __launch_bounds__(512) void dense_skinny_bf16_kernel(DenseParams p, i
         if (row >= p.M) continue;
         float g = ag[e], u = au[e];
         if (p.bias) { g += dn_ld((const bf16*)p.bias + nb); if (GATED) u += dn_ld((const bf16*)p.bias + nb + 32); }
-        g = dn_act(g, p.act);
-        dn_store<bf16>(p, row, oc, GATED ? g * u : g);
+        dn_store<bf16>(p, row, oc, GATED ? dn_gated(g, u, p.act, p.act_param) : dn_act(g, p.act));
     }
 }
 
@@ -471,16 +479,24 @@ __global__ __launch_bounds__(512) void dense_skinny_bf16_kernel(DenseParams p, i
 extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias,
                                   void* y, int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, float softcap,
                                   int32_t act_dtype, mi355_stream_t stream) {
+    return mi355_dense_linear_ex(x, ldx, M, w, N, K, bias, y, ldy, out_f32, gated, act, 0.f, softcap, act_dtype, stream);
+}
+
+// The same with a parameter for the activation.  act 5 (gated only): with L = act_param > 0, g' = min(gate, L), u' = clamp(up, -L, L) and
+// y = g' sigmoid(1.702 g') (u' + 1).
+extern "C" int mi355_dense_linear_ex(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias,
+                                     void* y, int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, float act_param, float softcap,
+                                     int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(x && w && y && M > 0 && N > 0 && K > 0 && ldx >= K, "dense_linear: M=%d N=%d K=%d ldx=%d", M, N, K, ldx);
     MI355_CHECK_ARG(act_dtype == MI355_ACT_BF16 || act_dtype == MI355_ACT_F32, "dense_linear: act_dtype=%d (bf16 or fp32)", act_dtype);
     MI355_CHECK_ARG(!gated || N % 64 == 0, "dense_linear: gated needs N %% 64 == 0 (N=%d)", N);
-    MI355_CHECK_ARG(act >= 0 && act <= 4, "dense_linear: act=%d", act);
+    MI355_CHECK_ARG(act >= 0 && act <= 5 && (act != DN_ACT_SWIGLU_CLAMP || (gated && act_param > 0.f)), "dense_linear: act=%d (gated=%d, parameter %g)", act, gated, (double)act_param);
     MI355_CHECK_ARG(ldy >= (gated ? N / 2 : N), "dense_linear: ldy=%d", ldy);
     const bool bf = act_dtype == MI355_ACT_BF16;
     const size_t es = bf ? 2 : 4;
     DenseParams p;
     p.x = x; p.w = w; p.bias = bias; p.y = y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.ldy = ldy;
-    p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = softcap;
+    p.gated = gated; p.act = act; p.act_param = act_param; p.out_f32 = bf ? out_f32 : 1; p.softcap = softcap;
     p.vec = (K % 8 == 0) && (ldx % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
     p.G = 1; p.xs = p.ws = p.ys = 0; p.offs = nullptr; p.gather = nullptr; p.tiles = nullptr; p.egate = nullptr; p.ldg = p.goff = 0;
     (void)es;
@@ -522,17 +538,26 @@ extern "C" int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const 
                                    int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, int32_t act_dtype, int32_t G, int64_t xs,
                                    int64_t ys, const int32_t* offs, const int32_t* gather, const int32_t* tiles, int32_t max_tiles,
                                    const float* egate, int32_t ldg, int32_t goff, mi355_stream_t stream) {
+    return mi355_dense_grouped_ex(x, ldx, M, w, N, K, bias, y, ldy, out_f32, gated, act, 0.f, act_dtype, G, xs, ys, offs, gather, tiles, max_tiles, egate, ldg,
+                                  goff, stream);
+}
+
+// The same with the activation's parameter (act 5 as in mi355_dense_linear_ex).
+extern "C" int mi355_dense_grouped_ex(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y,
+                                      int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, float act_param, int32_t act_dtype, int32_t G,
+                                      int64_t xs, int64_t ys, const int32_t* offs, const int32_t* gather, const int32_t* tiles, int32_t max_tiles,
+                                      const float* egate, int32_t ldg, int32_t goff, mi355_stream_t stream) {
     MI355_CHECK_ARG(x && w && y && M > 0 && N > 0 && K > 0 && G > 0 && xs >= 0 && ys >= 0, "dense_grouped: M=%d N=%d K=%d G=%d", M, N, K, G);
     MI355_CHECK_ARG(ldx >= xs * (G - 1) + K, "dense_grouped: ldx=%d for %d groups of K=%d at step %lld", ldx, G, K, (long long)xs);
     MI355_CHECK_ARG(act_dtype == MI355_ACT_BF16 || act_dtype == MI355_ACT_F32, "dense_grouped: act_dtype=%d (bf16 or fp32)", act_dtype);
     MI355_CHECK_ARG(!gated || N % 64 == 0, "dense_grouped: gated needs N %% 64 == 0 (N=%d)", N);
-    MI355_CHECK_ARG(act >= 0 && act <= 4, "dense_grouped: act=%d", act);
+    MI355_CHECK_ARG(act >= 0 && act <= 5 && (act != DN_ACT_SWIGLU_CLAMP || (gated && act_param > 0.f)), "dense_grouped: act=%d (gated=%d, parameter %g)", act, gated, (double)act_param);
     MI355_CHECK_ARG(ldy >= ys * (G - 1) + (gated ? N / 2 : N), "dense_grouped: ldy=%d", ldy);
     MI355_CHECK_ARG(G <= 65535 && (!gather || offs) && (!tiles || (offs && max_tiles > 0)), "dense_grouped: G=%d, gather and tiles need offs", G);
     const bool bf = act_dtype == MI355_ACT_BF16;
     DenseParams p;
     p.x = x; p.w = w; p.bias = bias; p.y = y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.ldy = ldy;
-    p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = 0.f;
+    p.gated = gated; p.act = act; p.act_param = act_param; p.out_f32 = bf ? out_f32 : 1; p.softcap = 0.f;
     p.vec = (K % 8 == 0) && (ldx % 8 == 0) && (xs % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
     p.G = G; p.xs = xs; p.ws = (long long)N * K; p.ys = ys; p.offs = offs; p.gather = gather; p.tiles = tiles;
     p.egate = egate; p.ldg = ldg; p.goff = goff;

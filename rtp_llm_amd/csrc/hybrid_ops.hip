@@ -166,6 +166,77 @@ __global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const f
     }
 }
 
+// ------------------------------------------------------------------------------------------------ scaled embedding; norm on a sublayer's OUTPUT
+// out[r] = table[ids[r]] * scale (fp32 stream); outh (null: none): the same rows rounded to the activation type, the input of the first sublayer of a
+// stack whose sublayers read the stream itself.
+template <typename T>
+__global__ __launch_bounds__(256) void hy_embed_scaled_kernel(const int32_t* ids, const T* table, int W, int vocab, float scale, float* out, T* outh) {
+    const int r = blockIdx.x;
+    int id = ids[r];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float v = (float)table[(size_t)id * W + c] * scale;
+        out[(size_t)r * W + c] = v;
+        if (outh) outh[(size_t)r * W + c] = (T)v;
+    }
+}
+
+__device__ __forceinline__ float hy_block_sum(float v, float* red) {       // red: 4 floats of LDS; every thread of the 256 calls it
+    v = hy_wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// A stack that norms what a sublayer RETURNS and lets the sublayers read the stream itself:  x[r] <- x[r] + N(y[r]) * w,  h[r] = x[r] rounded to
+// the activation type (the next sublayer's input; null: not written), with the sublayer's result
+//     y = ca * a + cb * b + sum_k ms.wts[r, k] * ms.y[ms.place[r, k]] + sigmoid(sg[r * ldsg]) * sh          (every term optional)
+// and N the layer norm (center: (y - mean) / sqrt(mean of squared deviations + eps)) or the RMS norm (y / sqrt(mean y^2 + eps)).
+// self_rows non-null: nothing is added; out row r is N(x[self_rows[r]]) * w in the activation type (the model's last norm on the asked rows).
+// Mean and variance are taken in two passes over the row kept in LDS; everything is fp32.
+struct BranchTerms { const float* a; float ca; const float* b; float cb; const float* sh; const float* sg; int ldsg; };
+
+template <typename T>
+__global__ __launch_bounds__(256) void hy_branch_norm_kernel(float* x, BranchTerms bt, MoeSum ms, const int32_t* self_rows, const T* w, int center, float eps,
+                                                             int W, T* h) {
+    extern __shared__ __attribute__((aligned(16))) float hy_xs[];
+    __shared__ float red[4];
+    const int r = blockIdx.x, src = self_rows ? self_rows[r] : r;
+    const size_t base = (size_t)src * W;
+    const float gsh = (bt.sh && bt.sg) ? hy_sigmoid(bt.sg[(size_t)src * bt.ldsg]) : 1.f;
+    float s1 = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float y;
+        if (self_rows) y = x[base + c];
+        else {
+            y = 0.f;
+            if (bt.a) y = bt.ca * bt.a[base + c];
+            if (bt.b) y = __builtin_fmaf(bt.cb, bt.b[base + c], y);
+            if (ms.y) {                    // the chosen experts in choice order
+                float sum = 0.f;
+                for (int k = 0; k < ms.top; ++k)
+                    sum = __builtin_fmaf(ms.wts[(size_t)src * ms.top + k], ms.y[(size_t)ms.place[(size_t)src * ms.top + k] * W + c], sum);
+                y += sum;
+            }
+            if (bt.sh) y = __builtin_fmaf(gsh, bt.sh[base + c], y);
+        }
+        hy_xs[c] = y;
+        s1 += y;
+    }
+    const float mean = center ? hy_block_sum(s1, red) / (float)W : 0.f;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) { const float d = hy_xs[c] - mean; ss = __builtin_fmaf(d, d, ss); }
+    const float inv = 1.f / sqrtf(hy_block_sum(ss, red) / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float n = (hy_xs[c] - mean) * inv * (float)w[c];
+        if (self_rows) { h[(size_t)r * W + c] = (T)n; continue; }
+        const float v = x[base + c] + n;
+        x[base + c] = v;
+        if (h) h[base + c] = (T)v;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ residual update + weighted average over depth + norm
 // A layer's own result X_n = x + a (a: the layer's last branch, may be null) joins the per-step stack of earlier results (stack[j] = X_j, planes
 // of `plane` floats; X_0 is the embedding output), and what the next layer reads is x <- sum_{j <= n} coef[j] X_j, summed in the order j = 0 .. n in
@@ -226,7 +297,8 @@ struct AttnGeom {
 
 // Optional steps around the rotation (AttnPrepExtra): a per-head RMS norm of queries and keys under weights shared by the heads (before the
 // rotation), a magnitude on cos and sin, and a position-dependent temperature on the queries, q *= 1 + coef ln(floor((p + 1) / every) + 1).
-struct AttnPrepExtra { const void* qnorm; const void* knorm; float mag; float qt_coef; int qt_every; };
+// norm_whole: the norm runs over ALL query heads of the row at once (and over all key heads), under weights [H * dim] / [G * dim].
+struct AttnPrepExtra { const void* qnorm; const void* knorm; float mag; float qt_coef; int qt_every; int norm_whole; };
 
 template <typename T>
 __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, int koff, int voff, AttnGeom g, const float* kfreq, const float* vfreq,
@@ -236,7 +308,25 @@ __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, i
     const int p = pos[r];
     float* row = qkv + (size_t)r * ld;
     const bool has_kv = kcache != nullptr;
-    if (ex.qnorm || (ex.knorm && has_kv)) {           // one wave per head: unit RMS over the head's channels, times the shared weight
+    if (ex.norm_whole && (ex.qnorm || (ex.knorm && has_kv))) {   // unit RMS over the whole projection (every head), times a weight per channel
+        __shared__ float redq[4], redk[4];
+        const int nq_ = ex.qnorm ? g.H * g.dim : 0, nk_ = (ex.knorm && has_kv) ? g.G * g.dim : 0;
+        float sq = 0.f, sk = 0.f;
+        for (int i = tid; i < nq_; i += 256) sq = __builtin_fmaf(row[i], row[i], sq);
+        for (int i = tid; i < nk_; i += 256) sk = __builtin_fmaf(row[koff + i], row[koff + i], sk);
+        sq = hy_wave_sum(sq); sk = hy_wave_sum(sk);
+        if ((tid & 63) == 0) { redq[tid >> 6] = sq; redk[tid >> 6] = sk; }
+        __syncthreads();
+        if (nq_) {
+            const float inv = 1.f / sqrtf(((redq[0] + redq[1]) + (redq[2] + redq[3])) / (float)nq_ + eps);
+            for (int i = tid; i < nq_; i += 256) row[i] = row[i] * inv * (float)((const T*)ex.qnorm)[i];
+        }
+        if (nk_) {
+            const float inv = 1.f / sqrtf(((redk[0] + redk[1]) + (redk[2] + redk[3])) / (float)nk_ + eps);
+            for (int i = tid; i < nk_; i += 256) row[koff + i] = row[koff + i] * inv * (float)((const T*)ex.knorm)[i];
+        }
+        __syncthreads();
+    } else if (ex.qnorm || (ex.knorm && has_kv)) {           // one wave per head: unit RMS over the head's channels, times the shared weight
         const int nqh = ex.qnorm ? g.H : 0, nkh = (ex.knorm && has_kv) ? g.G : 0;
         for (int j = tid >> 6; j < nqh + nkh; j += 4) {
             const bool isq = j < nqh;
@@ -760,7 +850,7 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
 // at a time: all threads compute the gates of the staged tokens once into LDS, then every thread walks the tokens in order (its RD rows:
 // decay, rank-one update, partial q . S), and the DS partial outputs per token are summed from LDS.  Short RD keeps the dependent chain per
 // token short; the walk itself is the sequential part of the recurrence.
-enum { SCAN_HGRN2 = 0, SCAN_GLA = 1, SCAN_FIXED = 2 };
+enum { SCAN_HGRN2 = 0, SCAN_GLA = 1, SCAN_FIXED = 2, SCAN_FIXED_SILU = 3 };
 
 struct ScanParams {
     const float* proj; int ld; int qo, ko, vo;     // fp32 projections [rows, ld]: q, k (GLA) or forget pre-activation (HGRN2), v at these columns
@@ -832,6 +922,8 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
                 const int hd = h * p.dim + d;
                 if (p.mode == SCAN_FIXED) {          // one decay per head (fp32 [H] behind `lower`), q and k as given
                     qv = rq[e]; kv = rk[e]; av = ((const float*)p.lower)[h];
+                } else if (p.mode == SCAN_FIXED_SILU) {   // the same decay; q, k (and v below) pass through silu first
+                    qv = hy_silu(rq[e]); kv = hy_silu(rk[e]); av = ((const float*)p.lower)[h];
                 } else if (p.mode == SCAN_HGRN2) {
                     const float lw = (float)((const T*)p.lower)[hd];
                     const float f = lw + (1.f - lw) * hy_sigmoid(rk[e] + (float)((const T*)p.fbias)[hd]);
@@ -847,10 +939,12 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
 #pragma unroll
         for (int e = 0; e < VE; ++e) {
             const int i = tid + e * blockDim.x;
-            if (i < nt * 64) v_s[i] = rv[e];
+            if (i < nt * 64) v_s[i] = p.mode == SCAN_FIXED_SILU ? hy_silu(rv[e]) : rv[e];
         }
-        for (int i = tid + VE * blockDim.x; i < nt * 64; i += blockDim.x)
-            v_s[i] = (v0 + (i & 63) < p.vdim) ? p.proj[(size_t)(t0 + (i >> 6)) * p.ld + p.vo + h * p.vdim + v0 + (i & 63)] : 0.f;
+        for (int i = tid + VE * blockDim.x; i < nt * 64; i += blockDim.x) {
+            const float vv = (v0 + (i & 63) < p.vdim) ? p.proj[(size_t)(t0 + (i >> 6)) * p.ld + p.vo + h * p.vdim + v0 + (i & 63)] : 0.f;
+            v_s[i] = p.mode == SCAN_FIXED_SILU ? hy_silu(vv) : vv;
+        }
         __syncthreads();
         if (t0 + TOK < r1) fetch(t0 + TOK);
         for (int t = 0; t < nt; ++t) {
@@ -1196,9 +1290,9 @@ __global__ __launch_bounds__(256) void hy_polynorm_kernel(const float* z, int ld
 }
 
 // ------------------------------------------------------------------------------------------------ mixture of experts: routing, sorting by expert, weighted sum
-// One wave per token: softmax over the E router logits (fp32); experts come in `groups` runs of E / groups neighbours, a group scores as its
-// best expert and only the `keep` best groups stay eligible; the `top` eligible experts with the largest scores are chosen, ties to the lower
-// index; the weights are their softmax scores as they are.
+// One wave per token: scores from the E router logits (fp32; softmax, or a sigmoid each); experts come in `groups` runs of E / groups neighbours, a
+// group scores as its best expert (or as the sum of its two best) and only the `keep` best groups stay eligible; the `top` eligible experts with
+// the largest scores are chosen, ties to the lower index; the weights are their scores as they are, times a constant.
 __device__ __forceinline__ void hy_wave_argmax(float& v, int& i) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -1208,36 +1302,47 @@ __device__ __forceinline__ void hy_wave_argmax(float& v, int& i) {
     }
 }
 
+// How a router scores: softmax over the logits or a sigmoid of each (sigmoid != 0); a group's score is its best expert's or the sum of its two
+// best (group_top = 1 | 2); the chosen experts weigh score * wscale.
+struct RouteMode { int sigmoid; int group_top; float wscale; };
+
 // The routing of one token by one wave; sc [E] and gb [groups] are the wave's scratch in LDS.  Every thread of the block calls it the same
 // number of times (it holds block barriers); a wave without a token passes active = false.
 __device__ __forceinline__ void hy_route_token(bool active, const float* zr, float* sc, float* gb, int E, int groups, int keep, int top, int32_t* ids,
-                                               float* wts, int lane) {
-    float m = -INFINITY;
-    if (active) for (int e = lane; e < E; e += 64) m = fmaxf(m, zr[e]);
-    m = hy_wave_max(m);
-    float sum = 0.f;
-    if (active) for (int e = lane; e < E; e += 64) { const float x = expf(zr[e] - m); sc[e] = x; sum += x; }
-    sum = hy_wave_sum(sum);
-    if (active) for (int e = lane; e < E; e += 64) sc[e] = sc[e] / sum;
+                                               float* wts, int lane, RouteMode rm) {
+    if (rm.sigmoid) {
+        if (active) for (int e = lane; e < E; e += 64) sc[e] = hy_sigmoid(zr[e]);
+    } else {
+        float m = -INFINITY;
+        if (active) for (int e = lane; e < E; e += 64) m = fmaxf(m, zr[e]);
+        m = hy_wave_max(m);
+        float sum = 0.f;
+        if (active) for (int e = lane; e < E; e += 64) { const float x = expf(zr[e] - m); sc[e] = x; sum += x; }
+        sum = hy_wave_sum(sum);
+        if (active) for (int e = lane; e < E; e += 64) sc[e] = sc[e] / sum;
+    }
     __syncthreads();
     const int per = E / groups;
     if (groups > 1 && keep < groups) {
         if (active)
             for (int g = lane; g < groups; g += 64) {
-                float b = -1.f;
-                for (int j = 0; j < per; ++j) b = fmaxf(b, sc[g * per + j]);
-                gb[g] = b;
+                float b1 = -1.f, b2 = -1.f;                       // the group's two largest scores (scores are >= 0)
+                for (int j = 0; j < per; ++j) {
+                    const float v = sc[g * per + j];
+                    if (v > b1) { b2 = b1; b1 = v; } else if (v > b2) b2 = v;
+                }
+                gb[g] = (rm.group_top >= 2 && per >= 2) ? b1 + b2 : b1;
             }
         __syncthreads();
-        for (int k = 0; k < keep; ++k) {          // the kept groups get a best score of 2 (above any probability), the others stay below
+        for (int k = 0; k < keep; ++k) {          // a kept group is marked by an infinite score, the others stay finite
             float bv = -2.f; int bi = 0x7fffffff;
-            if (active) for (int g = lane; g < groups; g += 64) { const float v = gb[g]; if (v <= 1.5f && (v > bv || (v == bv && g < bi))) { bv = v; bi = g; } }
+            if (active) for (int g = lane; g < groups; g += 64) { const float v = gb[g]; if (v < INFINITY && (v > bv || (v == bv && g < bi))) { bv = v; bi = g; } }
             hy_wave_argmax(bv, bi);
-            if (active && lane == 0) gb[bi] = 2.f;
+            if (active && lane == 0) gb[bi] = INFINITY;
             __syncthreads();
         }
     } else {
-        if (active) for (int g = lane; g < groups; g += 64) gb[g] = 2.f;
+        if (active) for (int g = lane; g < groups; g += 64) gb[g] = INFINITY;
         __syncthreads();
     }
     for (int k = 0; k < top; ++k) {
@@ -1245,18 +1350,18 @@ __device__ __forceinline__ void hy_route_token(bool active, const float* zr, flo
         if (active)
             for (int e = lane; e < E; e += 64) {
                 const float v = sc[e];
-                if (v >= 0.f && gb[e / per] > 1.5f && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }
+                if (v >= 0.f && gb[e / per] == INFINITY && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }
             }
         hy_wave_argmax(bv, bi);
-        if (active && lane == 0) { ids[k] = bi; wts[k] = bv; sc[bi] = -1.f; }     // taken
+        if (active && lane == 0) { ids[k] = bi; wts[k] = bv * rm.wscale; sc[bi] = -1.f; }     // taken
         __syncthreads();
     }
 }
 
-__global__ __launch_bounds__(64) void hy_moe_route_kernel(const float* z, int ld, int E, int groups, int keep, int top, int32_t* ids, float* wts) {
+__global__ __launch_bounds__(64) void hy_moe_route_kernel(const float* z, int ld, int E, int groups, int keep, int top, int32_t* ids, float* wts, RouteMode rm) {
     extern __shared__ float hy_rs[];            // scores [E], group best [groups]
     const int t = blockIdx.x;
-    hy_route_token(true, z + (size_t)t * ld, hy_rs, hy_rs + E, E, groups, keep, top, ids + (size_t)t * top, wts + (size_t)t * top, threadIdx.x);
+    hy_route_token(true, z + (size_t)t * ld, hy_rs, hy_rs + E, E, groups, keep, top, ids + (size_t)t * top, wts + (size_t)t * top, threadIdx.x, rm);
 }
 
 // Counting sort of the n = tokens * top (token, choice) pairs by expert, one block: offs [E + 1], src_row[sorted place] = token,
@@ -1293,7 +1398,7 @@ __global__ __launch_bounds__(1024) void hy_moe_align_kernel(const int32_t* ids, 
 
 // Routing and sorting of a few tokens (a decode step) in ONE block: its sixteen waves route a token each per trip, then the block sorts the pairs.
 __global__ __launch_bounds__(1024) void hy_moe_route_align_kernel(const float* z, int ld, int T, int E, int groups, int keep, int top, int32_t* ids, float* wts,
-                                                                  int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles) {
+                                                                  int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles, RouteMode rm) {
     extern __shared__ float hy_ra[];            // per wave: scores [E], group best [groups]; then counts [E], cursors [E]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float* sc = hy_ra + (size_t)wave * (E + groups);
@@ -1301,7 +1406,7 @@ __global__ __launch_bounds__(1024) void hy_moe_route_align_kernel(const float* z
         const int t = t0 + wave;
         const bool active = t < T;
         hy_route_token(active, z + (size_t)(active ? t : 0) * ld, sc, sc + E, E, groups, keep, top, ids + (size_t)(active ? t : 0) * top,
-                       wts + (size_t)(active ? t : 0) * top, lane);
+                       wts + (size_t)(active ? t : 0) * top, lane, rm);
     }
     __threadfence_block();
     __syncthreads();
@@ -1390,6 +1495,36 @@ extern "C" int mi355_hy_residual_norm(float* x, const float* a, const float* b, 
     return mi355_hy_gated_residual_norm(x, a, b, nullptr, 0, mult, rows, n, W, w1, w2, weight_offset, eps, h1, h2, nullptr, nullptr, nullptr, 0, act_dtype, stream);
 }
 
+// out fp32 [rows, W] = table[ids] * scale; outh (act_dtype [rows, W], or null): the same rows in the activation type.
+extern "C" int mi355_hy_embed_scaled(const int32_t* ids, int32_t rows, const void* table, int32_t W, int32_t vocab, float scale, float* out, void* outh,
+                                     int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(ids && table && out && rows > 0 && W > 0 && vocab > 0, "hy_embed_scaled: rows=%d W=%d", rows, W);
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_embed_scaled_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids, (const T*)table, W, vocab, scale, out,
+                                              (T*)outh));
+    MI355_CHECK_LAUNCH("hy_embed_scaled_kernel");
+    return MI355_OK;
+}
+
+// The end of a sublayer whose OUTPUT is normed: x [n, W] fp32 stream <- x + N(y) * w with y = ca * a + cb * b + (mixture sum) + sigmoid(sg) * sh, h [n, W]
+// (act_dtype, or null) = the new x.  a, b, sh: fp32 [n, W] or null; sg: fp32, one pre-activation per row at stride ldsg (null: sh is added as it is);
+// moe_*: as in mi355_hy_gated_residual_norm.  center != 0: layer norm (mean removed, variance of the deviations); 0: RMS norm.  w [W] of act_dtype.
+// self_rows (int32 [n]) non-null: no branch is read and x is not written; h [n, W] = N(x[self_rows]) * w.
+extern "C" int mi355_hy_branch_norm(float* x, const float* a, float ca, const float* b, float cb, const float* sh, const float* sg, int32_t ldsg,
+                                    const float* moe_y, const int32_t* moe_place, const float* moe_wts, int32_t moe_top, const int32_t* self_rows, int32_t n,
+                                    int32_t W, const void* w, int32_t center, float eps, void* h, int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(x && w && n > 0 && W > 0, "hy_branch_norm: n=%d W=%d", n, W);
+    MI355_CHECK_ARG(!moe_y || (moe_place && moe_wts && moe_top > 0), "hy_branch_norm: a mixture's sum needs its places and weights");
+    MI355_CHECK_ARG(self_rows ? h != nullptr : (a || b || sh || moe_y), "hy_branch_norm: nothing to norm");
+    MI355_CHECK_ARG(!sg || (sh && ldsg > 0), "hy_branch_norm: a gate without its branch (stride %d)", ldsg);
+    MI355_CHECK_ARG((size_t)W * 4 <= 64 * 1024, "hy_branch_norm: W=%d too wide for one block", W);
+    const BranchTerms bt{a, ca, b, cb, sh, sg, ldsg};
+    const MoeSum ms{moe_y, moe_place, moe_wts, moe_top};
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_branch_norm_kernel<T>, dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, bt, ms, self_rows, (const T*)w,
+                                              center, eps, W, (T*)h));
+    MI355_CHECK_LAUNCH("hy_branch_norm_kernel");
+    return MI355_OK;
+}
+
 // x fp32 [T, W] stream (the layer's input plus its earlier branches), a fp32 [T, W] or null; stack fp32 [>= n + 1, T, W] with planes 0 .. n - 1 filled;
 // coef fp32 [n + 1] on the device.  Writes stack[n] = x + a, x = sum_j coef[j] stack[j], h1 [rows_n, W] of act_dtype (null: no norm).  rows: null
 // (rows_n = T rows, in place), or rows_n row indices to form without writing x or the stack.
@@ -1426,9 +1561,19 @@ extern "C" int mi355_hy_attn_prep_ex(float* qkv, int32_t ld, int32_t koff, int32
                                      int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
                                      void* kcache, void* vcache, const void* qnorm, const void* knorm, float mag, float qt_coef, int32_t qt_every,
                                      int32_t act_dtype, mi355_stream_t stream) {
+    return mi355_hy_attn_prep_ex2(qkv, ld, koff, voff, geom, kfreq, vfreq, v_norm, eps, pos, seq, block_table, rows, kcache, vcache, qnorm, knorm, 0, mag, qt_coef,
+                                  qt_every, act_dtype, stream);
+}
+
+// norm_whole != 0: qnorm is [H * dim] and knorm [G * dim]; the queries of a row are brought to unit RMS over all their heads at once (the keys likewise)
+// and multiplied by a weight per channel, before the rotation.
+extern "C" int mi355_hy_attn_prep_ex2(float* qkv, int32_t ld, int32_t koff, int32_t voff, const int32_t* geom, const float* kfreq, const float* vfreq,
+                                      int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
+                                      void* kcache, void* vcache, const void* qnorm, const void* knorm, int32_t norm_whole, float mag, float qt_coef,
+                                      int32_t qt_every, int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(qkv && geom && pos && seq && rows > 0, "hy_attn_prep: null argument");
     MI355_CHECK_ARG(qt_coef == 0.f || qt_every > 0, "hy_attn_prep: query temperature every %d positions", qt_every);
-    const AttnPrepExtra ex{qnorm, knorm, mag, qt_coef, qt_every};
+    const AttnPrepExtra ex{qnorm, knorm, mag, qt_coef, qt_every, norm_whole};
     const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
     MI355_CHECK_ARG((g.rot_dims == 0 || kfreq) && (!kcache || (vcache && block_table)), "hy_attn_prep: missing table or cache");
@@ -1511,6 +1656,7 @@ extern "C" int mi355_hy_attn_tiles_ex(const float* q, int32_t ldq, float scale, 
 // mode 0 (HGRN2): q = silu(proj q), f = lower + (1 - lower) sigmoid(proj k + fbias), a = f, k = 1 - f.
 // mode 1 (GLA):   q = proj q * qscale, k = proj k, a = sigmoid(z)^(1 / tau).
 // mode 2 (fixed): q = proj q, k = proj k, a = lower[h] (fp32 [H], one decay per head whatever act_dtype is).
+// mode 3 (fixed, silu): q = silu(proj q), k = silu(proj k), v = silu(proj v), a = lower[h] as in mode 2.
 // Sequence s owns rows row_start[s] .. row_start[s + 1] - 1 in order, continues the state in slot[s] (starts from zero when first_pos[s] == 0)
 // and leaves the new state there.  out fp32 [rows, H * vdim].
 extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_t qo, int32_t ko, int32_t vo, const float* z, int32_t ldz,
@@ -1518,7 +1664,7 @@ extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_
                              const int32_t* row_start, const int32_t* slot, const int32_t* first_pos, int32_t nseq, float* state, float* out,
                              int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(proj && row_start && slot && first_pos && state && out && nseq > 0 && H > 0 && dim > 0 && vdim > 0, "hy_scan: bad argument");
-    MI355_CHECK_ARG(mode == SCAN_HGRN2 ? (lower && fbias) : mode == SCAN_FIXED ? lower != nullptr : (mode == SCAN_GLA && z && tau > 0.f),
+    MI355_CHECK_ARG(mode == SCAN_HGRN2 ? (lower && fbias) : (mode == SCAN_FIXED || mode == SCAN_FIXED_SILU) ? lower != nullptr : (mode == SCAN_GLA && z && tau > 0.f),
                     "hy_scan: mode %d lacks its gate inputs", mode);
     MI355_CHECK_ARG(dim <= 512, "hy_scan: key size %d > 512", dim);
     const int RD = dim <= 128 ? 8 : dim <= 256 ? 16 : 32;       // rows per thread: at most 16 groups of RD rows (1024 threads)
@@ -1614,11 +1760,20 @@ extern "C" int mi355_hy_polynorm(const float* z, int32_t ld, int32_t rows, int32
 // z fp32 [tokens, ld] router logits -> ids int32 [tokens, top], wts fp32 [tokens, top]
 extern "C" int mi355_hy_moe_route(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
                                   mi355_stream_t stream) {
+    return mi355_hy_moe_route_ex(z, ld, tokens, E, groups, keep, top, ids, wts, 0, 1, 1.f, stream);
+}
+
+// The same with the router's form as arguments: score_sigmoid (scores are sigmoids of the logits instead of their softmax), group_top (1: a group
+// scores as its best expert; 2: as the sum of its two best), wscale (the chosen experts weigh score * wscale).
+extern "C" int mi355_hy_moe_route_ex(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
+                                     int32_t score_sigmoid, int32_t group_top, float wscale, mi355_stream_t stream) {
+    MI355_CHECK_ARG(group_top == 1 || group_top == 2, "hy_moe_route: a group scores by its best %d experts (1 or 2)", group_top);
+    const RouteMode rm{score_sigmoid, group_top, wscale};
     MI355_CHECK_ARG(z && ids && wts && tokens > 0 && E > 0 && ld >= E, "hy_moe_route: tokens=%d experts=%d", tokens, E);
     MI355_CHECK_ARG(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top >= 1 && top <= (E / groups) * keep, "hy_moe_route: %d experts in %d groups, keep %d, top %d",
                     E, groups, keep, top);
     MI355_CHECK_ARG((size_t)(E + groups) * 4 <= 48 * 1024, "hy_moe_route: %d experts do not fit the block's scratch", E);
-    hipLaunchKernelGGL(hy_moe_route_kernel, dim3(tokens), dim3(64), (size_t)(E + groups) * 4, (hipStream_t)stream, z, ld, E, groups, keep, top, ids, wts);
+    hipLaunchKernelGGL(hy_moe_route_kernel, dim3(tokens), dim3(64), (size_t)(E + groups) * 4, (hipStream_t)stream, z, ld, E, groups, keep, top, ids, wts, rm);
     MI355_CHECK_LAUNCH("hy_moe_route_kernel");
     return MI355_OK;
 }
@@ -1635,6 +1790,14 @@ extern "C" int mi355_hy_moe_align(const int32_t* ids, int32_t n, int32_t top, in
 // Both in one launch for a few tokens (tokens <= 64 and the scratch of sixteen waves fits: MI355_ERR_UNSUPPORTED otherwise).
 extern "C" int mi355_hy_moe_route_align(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
                                         int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles, mi355_stream_t stream) {
+    return mi355_hy_moe_route_align_ex(z, ld, tokens, E, groups, keep, top, ids, wts, offs, src_row, place_of, tiles, 0, 1, 1.f, stream);
+}
+
+extern "C" int mi355_hy_moe_route_align_ex(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids,
+                                           float* wts, int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles, int32_t score_sigmoid,
+                                           int32_t group_top, float wscale, mi355_stream_t stream) {
+    MI355_CHECK_ARG(group_top == 1 || group_top == 2, "hy_moe_route_align: a group scores by its best %d experts (1 or 2)", group_top);
+    const RouteMode rm{score_sigmoid, group_top, wscale};
     MI355_CHECK_ARG(z && ids && wts && offs && src_row && place_of && tiles && tokens > 0 && E > 0 && ld >= E, "hy_moe_route_align: tokens=%d experts=%d", tokens, E);
     MI355_CHECK_ARG(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top >= 1 && top <= (E / groups) * keep, "hy_moe_route_align: %d experts in %d groups, keep %d, top %d",
                     E, groups, keep, top);
@@ -1643,7 +1806,7 @@ extern "C" int mi355_hy_moe_route_align(const float* z, int32_t ld, int32_t toke
         mi355_set_error("hy_moe_route_align: %d tokens, %d experts: use the two launches", tokens, E);
         return MI355_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(hy_moe_route_align_kernel, dim3(1), dim3(1024), lds, (hipStream_t)stream, z, ld, tokens, E, groups, keep, top, ids, wts, offs, src_row, place_of, tiles);
+    hipLaunchKernelGGL(hy_moe_route_align_kernel, dim3(1), dim3(1024), lds, (hipStream_t)stream, z, ld, tokens, E, groups, keep, top, ids, wts, offs, src_row, place_of, tiles, rm);
     MI355_CHECK_LAUNCH("hy_moe_route_align_kernel");
     return MI355_OK;
 }

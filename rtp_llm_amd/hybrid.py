@@ -15,7 +15,12 @@ l<i>.mlp.{up, down, act} or l<i>.mlp.{router, e<j>.{gate, up, down}, shared.{gat
 x <- x + mixer(norm1 x), x <- x + mlp(norm2 x) whose norms have ONE gain for all channels, every layer reading a learned weighted average
 of the embedding output and the results of all layers before it (l<i>.dwa); a hashed bigram table beside the token embedding (bigram);
 mixers: a generalized delta-rule recurrence, causal attention with a query temperature, a score cap, biases and per-head output gates, and
-sliding-window attention with normed, YaRN-rotated queries and keys; gelu-gated MLPs)."""
+sliding-window attention with normed, YaRN-rotated queries and keys; gelu-gated MLPs) and Nudorax (layers x <- x + LN(mixer(x)),
+x <- x + LN(mlp(x)): the sublayers read the stream itself and a layer norm follows each; every mixer is two side by side, windowed attention
+with a learned sink and queries / keys normed over all heads at once beside lightning attention; mixtures of clamped gated experts under a
+sigmoid router whose groups rank by their two best, with a gated shared expert; the embedding is scaled on entry and is the output head;
+checkpoint tensors l<i>.mix.left.{q, k, v, q.norm, k.norm, sink, o}, l<i>.mix.right.{q, k, v, g, norm, o}, l<i>.mlp.{router, e<j>.*, shared.{gate, up,
+down, sg}})."""
 import json
 import os
 from dataclasses import dataclass, field
@@ -25,18 +30,31 @@ import torch
 
 from . import hybrid_ops as hops
 from .mixers import (AttentionSpec, DeltaRuleSpec, GatedLinearRecurrence, GatedMLP, GeneralizedDeltaRule, LatentAttention, LatentAttentionSpec,
-                     PagedChunkAttention, PolyNormMLP, RecurrenceSpec, Retention, RetentionSpec, RotarySpec, RoutedExperts, RouterSpec, StepBatch)
+                     LightningAttention, LightningSpec, PagedChunkAttention, ParallelMixer, PolyNormMLP, RecurrenceSpec, Retention, RetentionSpec,
+                     RotarySpec, RoutedExperts, RouterSpec, StepBatch)
+
+
+@dataclass
+class ParallelSpec:
+    """Two mixers on the same input, added as left_scale * left + right_scale * right; their checkpoint tensors sit under mix.left. / mix.right."""
+    left: Union[AttentionSpec, LightningSpec]
+    right: Union[AttentionSpec, LightningSpec]
+    left_scale: float = 1.0
+    right_scale: float = 1.0
 
 
 @dataclass
 class HybridLayerSpec:
-    kind: str                                        # "attention" | "hgrn2" | "gla" | "latent_attention" | "retention" | "delta_rule"
-    mixer: Union[AttentionSpec, RecurrenceSpec, LatentAttentionSpec, RetentionSpec, DeltaRuleSpec]
+    kind: str                                        # "attention" | "hgrn2" | "gla" | "latent_attention" | "retention" | "delta_rule" | "lightning" | "parallel"
+    mixer: Union[AttentionSpec, RecurrenceSpec, LatentAttentionSpec, RetentionSpec, DeltaRuleSpec, LightningSpec, ParallelSpec]
     ff: Optional[int] = None                         # None: the layer has no MLP; hidden size of the dense MLP or of one routed expert
     mlp_act: str = "relu"
     mlp_kind: str = "gated"                          # "gated" | "polynorm" | "experts"
     router: Optional[RouterSpec] = None              # experts: the router ...
     shared_ff: Optional[int] = None                  # ... and the hidden size of the expert every token runs (None: no such expert)
+    act_param: float = 0.0                           # parameter of mlp_act (the limit of "swiglu_clamp") ...
+    shared_act_param: float = 0.0                    # ... and the shared expert's own
+    shared_gate: bool = False                        # the shared expert's output is multiplied by sigmoid(w . h), one number per token (mlp.shared.sg)
 
 
 @dataclass
@@ -64,6 +82,10 @@ class HybridConfig:
     scalar_norm: bool = False                        # every norm's weight is ONE number for all channels
     depth_mix: bool = False                          # a layer reads sum_j dwa[j] X_j over the embedding output X_0 and all earlier layers' results
     bigram: Optional[BigramSpec] = None              # hashed (previous token, token) rows added to the token embedding
+    embed_scale: float = 1.0                         # the embedding rows are multiplied by this as they enter the stream
+    tied_head: bool = False                          # the output head is the embedding table itself (without embed_scale); no `head` tensor
+    out_norm: bool = False                           # sequential layers whose sublayers read the stream ITSELF and whose OUTPUT is normed: x <- x + norm(f(x))
+    norm_kind: str = "rms"                           # "rms" | "layer" (mean removed, variance of the deviations, a weight and no bias)
 
     @staticmethod
     def from_json(cfg: dict) -> "HybridConfig":
@@ -179,7 +201,47 @@ def nepudra_from_json(cfg: dict) -> HybridConfig:
                         bigram=BigramSpec(int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"])) if bg else None)
 
 
-_READERS = {"nufalorn": HybridConfig.nufalorn_from_json, "pokepel": HybridConfig.pokepel_from_json, "nepudra": nepudra_from_json}
+def nudorax_from_json(cfg: dict) -> HybridConfig:
+    """The Nudorax reading of config.json.  Layer type "parallel": mixer.{left, right, left_scale, right_scale} with left = windowed attention
+    {heads, kv_heads, dim, vdim, scale, mask.size, rot.{dims, base, scaling.{factor, low, high, original}}} (queries and keys normed over all heads
+    at once, rotary pairs half a span apart with wavelength-scaled steps, a learned sink logit per head) and right = lightning attention
+    {heads, dim, vdim, decay[heads]}.  mlp: null or {kind: moe, expert.{ff, limit}, router.{experts, top, scale, groups.{count, keep}},
+    shared.{ff, limit}} with a sigmoid router whose groups rank by their two best experts, clamped gated experts and a gated shared expert.
+    Layer norms on the sublayers' outputs, the embedding scaled on entry and reused as the output head, a tanh cap on the logits."""
+    def attention(mx):
+        mask = mx.get("mask") or {}
+        return AttentionSpec(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads") or mx["heads"]), dim=int(mx["dim"]), vdim=int(mx.get("vdim") or mx["dim"]),
+                             scale=float(mx["scale"]), rot=RotarySpec.from_json(mx.get("rot"), "halves", scaling="wavelength"),
+                             window=int(mask.get("size") or 0), sink=True, learned_sink=True, qk_norm=True, qk_norm_whole=True)
+
+    def lightning(mx):
+        return LightningSpec(heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx.get("vdim") or mx["dim"]), decay=tuple(float(a) for a in mx["decay"]))
+
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        kind, mx, mlp = L["type"], L["mixer"], L.get("mlp")
+        if kind != "parallel":
+            raise NotImplementedError(f"layer {i}: mixer type {kind!r}")
+        if len(mx["right"]["decay"]) != int(mx["right"]["heads"]):
+            raise ValueError(f"layer {i}: {len(mx['right']['decay'])} decays for {mx['right']['heads']} heads")
+        spec = ParallelSpec(attention(mx["left"]), lightning(mx["right"]), float(mx.get("left_scale", 1.0)), float(mx.get("right_scale", 1.0)))
+        if mlp is None:
+            layers.append(HybridLayerSpec(kind, spec))
+        elif mlp.get("kind") == "moe":
+            r, sh = mlp["router"], mlp.get("shared")
+            grp = r.get("groups") or {}
+            count = int(grp.get("count", 1))
+            router = RouterSpec(int(r["experts"]), int(r["top"]), count, int(grp.get("keep", count)), score="sigmoid", group_top=2, scale=float(r.get("scale", 1.0)))
+            layers.append(HybridLayerSpec(kind, spec, int(mlp["expert"]["ff"]), "swiglu_clamp", "experts", router, None if not sh else int(sh["ff"]),
+                                          act_param=float(mlp["expert"]["limit"]), shared_act_param=float(sh["limit"]) if sh else 0.0, shared_gate=bool(sh)))
+        else:
+            raise NotImplementedError(f"layer {i}: mlp kind {mlp.get('kind')!r}")
+    return HybridConfig(name=str(cfg["architecture"]), vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=layers, eps=float(cfg["norm"]["eps"]),
+                        logit_softcap=float(cfg.get("logit_softcap") or 0.0), norm_offset=0.0, sequential=True, out_norm=True, norm_kind="layer",
+                        embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)), tied_head=True)
+
+
+_READERS = {"nufalorn": HybridConfig.nufalorn_from_json, "pokepel": HybridConfig.pokepel_from_json, "nepudra": nepudra_from_json, "nudorax": nudorax_from_json}
 
 
 class HybridModel:
@@ -203,7 +265,7 @@ class HybridModel:
             return t.reshape(1).expand(cfg.width).contiguous() if cfg.scalar_norm else t
 
         self.embed = get("embed")
-        self.head = get("head")
+        self.head = self.embed if cfg.tied_head else get("head")
         self.final_norm = norm_w("final.norm")
         self.bigram = None
         if cfg.bigram is not None:
@@ -223,12 +285,30 @@ class HybridModel:
         self.n_mix = {}                                  # layer -> (columns, padded columns) of the mixer's inputs inside the layer's shared linear
         for i, L in enumerate(cfg.layers):
             p = f"l{i}."
-            if L.kind == "attention":
-                a, own = L.mixer, L.mixer.kv_from is None
+            def attention(a, q):
+                own = a.kv_from is None
                 names = ["q", "o"] + (["k", "v"] if own else []) + (["g"] if a.out_gate else []) + (["o.b"] if a.out_bias else [])
                 names += (["q.b"] + (["k.b", "v.b"] if own else [])) if a.bias else []
                 names += (["q.norm"] + (["k.norm"] if own else [])) if a.qk_norm else []
-                mixer = PagedChunkAttention(a, sub(p + "mix.", names), cfg.eps, page, self.device)
+                names += ["sink"] if a.sink and a.learned_sink else []
+                return PagedChunkAttention(a, sub(q, names), cfg.eps, page, self.device)
+
+            def lightning(a, q):
+                return LightningAttention(a, sub(q, ["q", "k", "v", "g", "norm", "o"]), cfg.eps, self.device)
+
+            def side(a, q):
+                if isinstance(a, AttentionSpec):
+                    if a.kv_from is not None:
+                        raise NotImplementedError("a side of a parallel mixer keeps its own keys and values")
+                    return attention(a, q)
+                return lightning(a, q)
+
+            if L.kind == "attention":
+                mixer = attention(L.mixer, p + "mix.")
+            elif L.kind == "lightning":
+                mixer = lightning(L.mixer, p + "mix.")
+            elif L.kind == "parallel":
+                mixer = ParallelMixer(side(L.mixer.left, p + "mix.left."), side(L.mixer.right, p + "mix.right."), L.mixer.left_scale, L.mixer.right_scale)
             elif L.kind == "delta_rule":
                 mixer = GeneralizedDeltaRule(L.mixer, sub(p + "mix.", ["r", "k", "v", "a", "a.b", "g", "w1", "w2", "w0", "norm", "o"]), cfg.eps)
             elif L.kind == "latent_attention":
@@ -241,7 +321,7 @@ class HybridModel:
                 mixer = GatedLinearRecurrence(L.mixer, sub(p + "mix.", ["q", "k", "v", "g", "a1", "a2", "a2.b", "norm", "o"]), cfg.eps)
             mlp = None
             if L.ff is not None:
-                gated = lambda q, act: GatedMLP(get(q + "gate"), get(q + "up"), get(q + "down"), act)
+                gated = lambda q, act, par=0.0: GatedMLP(get(q + "gate"), get(q + "up"), get(q + "down"), act, par)
                 if L.mlp_kind == "gated":
                     mlp = gated(p + "mlp.", L.mlp_act)
                 elif L.mlp_kind == "polynorm":
@@ -249,7 +329,9 @@ class HybridModel:
                 else:
                     ex = [p + f"mlp.e{j}." for j in range(L.router.experts)]
                     mlp = RoutedExperts(L.router, get(p + "mlp.router"), [get(q + "gate") for q in ex], [get(q + "up") for q in ex],
-                                        [get(q + "down") for q in ex], gated(p + "mlp.shared.", L.mlp_act) if L.shared_ff is not None else None, L.mlp_act)
+                                        [get(q + "down") for q in ex],
+                                        gated(p + "mlp.shared.", L.mlp_act, L.shared_act_param or L.act_param) if L.shared_ff is not None else None, L.mlp_act,
+                                        act_param=L.act_param, shared_gate=get(p + "mlp.shared.sg") if L.shared_gate else None)
             gate_w = gate_b = None
             if cfg.branch_gates:                       # both gates in one linear: columns [0, W) scale the mixer, [W, 2W) the MLP
                 names = ["rg1"] + (["rg2"] if mlp is not None else [])
@@ -274,13 +356,19 @@ class HybridModel:
                 mixer.w_in = None                      # lives on as the leading rows of the shared weight
             self.layers.append((L, mixer, mlp, norm_w(p + "norm1"), n2, gate_w, gate_b))
         self.has_state = any(L.kind not in ("attention", "latent_attention") for L in cfg.layers)
+        self.norm_center = cfg.norm_kind == "layer"
+        if cfg.norm_kind not in ("rms", "layer") or (cfg.norm_kind == "layer" and not cfg.out_norm):
+            raise NotImplementedError(f"norm kind {cfg.norm_kind!r} (layer norms are built for stacks that norm the sublayers' outputs)")
 
     # ---- what an engine has to allocate
     def cache_layout(self):
-        """Per layer: ("kv", K page shape, V page shape) | ("kv_from", layer) | ("latent", page shape) | ("state", per-slot shape)."""
+        """Per layer: ("kv", K page shape, V page shape) | ("kv_from", layer) | ("latent", page shape) | ("state", per-slot shape) |
+        ("sides", [entries of the two sides of a parallel mixer, each "kv" or "state"])."""
         out = []
         for L, mixer, *_ in self.layers:
-            if L.kind == "attention":
+            if L.kind == "parallel":
+                out.append(("sides", [(("kv",) + m.cache_shapes()) if m.cache_kind() == "kv" else ("state", m.state_shape()) for m in (mixer.left, mixer.right)]))
+            elif L.kind == "attention":
                 out.append((("kv",) + mixer.cache_shapes()) if mixer.owns_cache else ("kv_from", L.mixer.kv_from))
             elif L.kind == "latent_attention":
                 out.append(("latent", mixer.cache_shape()))
@@ -289,10 +377,18 @@ class HybridModel:
         return out
 
     def alloc_cache(self, num_pages: int, num_slots: int):
-        """Cache tensors for `num_pages` pages and `num_slots` state slots: per layer (kcache, vcache) or a state tensor."""
+        """Cache tensors for `num_pages` pages and `num_slots` state slots: per layer (kcache, vcache) or a state tensor; for a parallel mixer
+        the tuple of its sides' tensors in order."""
         caches = []
+        pages = lambda shape: torch.zeros(num_pages, *shape, dtype=self.dtype, device=self.device)
+        slots = lambda shape: torch.zeros(num_slots, *shape, dtype=torch.float32, device=self.device)
         for ent in self.cache_layout():
-            if ent[0] == "kv":
+            if ent[0] == "sides":
+                flat = []
+                for e in ent[1]:
+                    flat += [pages(e[1]), pages(e[2])] if e[0] == "kv" else [slots(e[1])]
+                caches.append(tuple(flat))
+            elif ent[0] == "kv":
                 caches.append((torch.zeros(num_pages, *ent[1], dtype=self.dtype, device=self.device),
                                torch.zeros(num_pages, *ent[2], dtype=self.dtype, device=self.device)))
             elif ent[0] == "kv_from":
@@ -308,6 +404,8 @@ class HybridModel:
         """fp32 logits [len(batch.want), vocab] of the wanted rows; the caches of every row's sequence are advanced.  collect: receives
         the residual stream after every layer (debugging / tests; costs one extra norm launch per layer)."""
         cfg = self.cfg
+        if cfg.out_norm:
+            return self._forward_out_norm(batch, caches, collect)
         if cfg.sequential:
             return self._forward_sequential(batch, caches, collect)
         x = hops.embed(batch.tokens, self.embed)
@@ -373,6 +471,28 @@ class HybridModel:
         if collect is not None:
             h1, _ = hops.residual_norm(x, None, None, 1.0, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset, rows=batch.want)
         return hops.dense_linear(h1, self.head, out_dtype=torch.float32, softcap=cfg.logit_softcap)
+
+
+    def _forward_out_norm(self, batch: StepBatch, caches, collect: Optional[list]) -> torch.Tensor:
+        """The step of a member whose sublayers read the stream itself and whose outputs are normed: x <- x + N(mixer(x)), x <- x + N(mlp(x)).  The
+        stream stays fp32; the sublayers' input is its rounding to the activation type, written by the kernel that ends the sublayer before.  A
+        parallel mixer's two outputs and a mixture's parts (chosen experts, gated shared expert) are summed inside that kernel."""
+        cfg = self.cfg
+        lowp = self.dtype != torch.float32
+        x, h = hops.embed_scaled(batch.tokens, self.embed, cfg.embed_scale, rounded=lowp)
+        for (L, mixer, mlp, n1, n2, _gw, _gb), cache in zip(self.layers, caches):
+            src = h if lowp else x
+            out = mixer.forward(src, batch, *cache) if isinstance(cache, tuple) else mixer.forward(src, batch, cache)
+            a, ca, b, cb = out if isinstance(out, tuple) else (out, 1.0, None, 1.0)
+            h = hops.branch_norm(x, n1, cfg.eps, a=a, ca=ca, b=b, cb=cb, center=self.norm_center, rounded=lowp)
+            if mlp is not None:
+                src = h if lowp else x
+                y = mlp.forward(src, defer=True) if isinstance(mlp, RoutedExperts) else mlp.forward(src)
+                h = hops.branch_norm(x, n2, cfg.eps, center=self.norm_center, rounded=lowp, **({"moe": y} if isinstance(y, hops.MoeSum) else {"a": y}))
+            if collect is not None:
+                collect.append(x.clone())
+        hf = hops.norm_rows(x, batch.want, self.final_norm, cfg.eps, center=self.norm_center)
+        return hops.dense_linear(hf, self.head, out_dtype=torch.float32, softcap=cfg.logit_softcap)
 
 
 def load_hybrid_checkpoint(path: str, dtype: torch.dtype, device, page: int = 64) -> HybridModel:

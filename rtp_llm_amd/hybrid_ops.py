@@ -9,9 +9,9 @@ import torch
 
 from . import _C
 
-ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU_TANH, ACT_TANH = 0, 1, 2, 3, 4
-ACTIVATIONS = {"none": ACT_NONE, "relu": ACT_RELU, "silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH, "tanh": ACT_TANH}
-SCAN_HGRN2, SCAN_GLA, SCAN_FIXED = 0, 1, 2
+ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU_TANH, ACT_TANH, ACT_SWIGLU_CLAMP = 0, 1, 2, 3, 4, 5
+ACTIVATIONS = {"none": ACT_NONE, "relu": ACT_RELU, "silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH, "tanh": ACT_TANH, "swiglu_clamp": ACT_SWIGLU_CLAMP}
+SCAN_HGRN2, SCAN_GLA, SCAN_FIXED, SCAN_FIXED_SILU = 0, 1, 2, 3
 LAYOUTS = {"interleaved": 0, "halves": 1}
 
 
@@ -46,10 +46,11 @@ def _rows(t: torch.Tensor, name: str) -> int:
 
 
 def dense_linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, *, out_dtype: Optional[torch.dtype] = None,
-                 gated: bool = False, act: int = ACT_NONE, softcap: float = 0.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 gated: bool = False, act: int = ACT_NONE, softcap: float = 0.0, out: Optional[torch.Tensor] = None, act_param: float = 0.0) -> torch.Tensor:
     """y = x @ w.T (+ bias) for w [N, K] in checkpoint layout.  gated: w holds groups of 32 gate rows followed by the 32 up rows of the
     same channels and y [M, N / 2] = act(gate) * up; without `gated`, act applies to the plain output.  out_dtype float32 keeps the accumulator;
-    softcap > 0 applies cap * tanh(y / cap)."""
+    softcap > 0 applies cap * tanh(y / cap).  ACT_SWIGLU_CLAMP (gated only) with L = act_param: g = min(gate, L), u = clamp(up, -L, L),
+    y = g sigmoid(1.702 g) (u + 1)."""
     _dev(x, w.dtype, "dense_linear.x"); _dev(w, w.dtype, "dense_linear.w")
     ldx = _rows(x, "dense_linear.x")
     M, K = x.shape
@@ -77,9 +78,9 @@ def dense_linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] 
     ldy = _rows(out, "dense_linear.out")
     if M == 0:
         return out
-    _C.check_hybrid(_C.hybrid_lib().mi355_dense_linear(x.data_ptr(), ldx, M, w.data_ptr(), N, K, _p(bias), out.data_ptr(), ldy,
-                                                       1 if od == torch.float32 else 0, 1 if gated else 0, act, float(softcap),
-                                                       act_code(w.dtype), _stream()), "dense_linear")
+    _C.check_hybrid(_C.hybrid_lib().mi355_dense_linear_ex(x.data_ptr(), ldx, M, w.data_ptr(), N, K, _p(bias), out.data_ptr(), ldy,
+                                                          1 if od == torch.float32 else 0, 1 if gated else 0, act, float(act_param), float(softcap),
+                                                          act_code(w.dtype), _stream()), "dense_linear")
     return out
 
 
@@ -116,6 +117,71 @@ def embed(ids: torch.Tensor, table: torch.Tensor, *, prev: Optional[torch.Tensor
     return out
 
 
+def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float, *, rounded: bool = False):
+    """(fp32 stream rows [T, W] = table[ids] * scale, the same rows in the table's dtype or None): `rounded` asks for the second tensor, the input
+    of the first sublayer of a stack whose sublayers read the stream itself."""
+    _dev(ids, torch.int32, "embed_scaled.ids")
+    T, W = ids.numel(), table.shape[1]
+    out = torch.empty(T, W, dtype=torch.float32, device=table.device)
+    outh = torch.empty(T, W, dtype=table.dtype, device=table.device) if rounded else None
+    if T:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_embed_scaled(ids.data_ptr(), T, table.data_ptr(), W, table.shape[0], float(scale), out.data_ptr(), _p(outh),
+                                                              act_code(table.dtype), _stream()), "hy_embed_scaled")
+    return out, outh
+
+
+def branch_norm(x: torch.Tensor, w: torch.Tensor, eps: float, *, a: Optional[torch.Tensor] = None, ca: float = 1.0, b: Optional[torch.Tensor] = None,
+                cb: float = 1.0, moe: Optional["MoeSum"] = None, center: bool = True, rounded: bool = False) -> Optional[torch.Tensor]:
+    """The end of a sublayer whose OUTPUT is normed: x <- x + N(y) * w in place on the fp32 stream, y = ca * a + cb * b + the mixture sum `moe`
+    (its `extra` is the shared expert's output, multiplied by sigmoid(moe.extra_gate) per row when that is given).  N: layer norm (center) or RMS
+    norm.  -> the new rows in w's dtype when `rounded`, else None."""
+    _dev(x, torch.float32, "branch_norm.x")
+    T, W = x.shape
+    if not x.is_contiguous() or w.numel() != W or not w.is_contiguous():
+        raise _C.Mi355Error(f"branch_norm: stream {tuple(x.shape)} (contiguous) against a weight {tuple(w.shape)}")
+    sh = sg = None
+    ldsg = 0
+    if moe is not None:
+        _dev(moe.y, torch.float32, "branch_norm.moe.y"); _dev(moe.wts, torch.float32, "branch_norm.moe.wts"); _dev(moe.place_of, torch.int32, "branch_norm.moe.place")
+        if moe.wts.shape[0] != T or moe.y.shape != (moe.wts.numel(), W) or moe.place_of.numel() != moe.wts.numel() or not (moe.y.is_contiguous() and moe.wts.is_contiguous()):
+            raise _C.Mi355Error(f"branch_norm: mixture sum y {tuple(moe.y.shape)} wts {tuple(moe.wts.shape)} against the stream {tuple(x.shape)}")
+        sh, sg = moe.extra, getattr(moe, "extra_gate", None)
+        if sg is not None:
+            _dev(sg, torch.float32, "branch_norm.moe.extra_gate")
+            if sh is None or sg.dim() != 1 or sg.numel() != T:
+                raise _C.Mi355Error(f"branch_norm: gate {tuple(sg.shape)} of the shared branch for {T} rows")
+            ldsg = sg.stride(0)
+    for t, nm in ((a, "a"), (b, "b"), (sh, "shared")):
+        if t is not None:
+            _dev(t, torch.float32, "branch_norm." + nm)
+            if t.shape != x.shape or not t.is_contiguous():
+                raise _C.Mi355Error(f"branch_norm.{nm}: {tuple(t.shape)} against the stream {tuple(x.shape)}")
+    if a is None and b is None and moe is None:
+        raise _C.Mi355Error("branch_norm: no branch")
+    h = torch.empty(T, W, dtype=w.dtype, device=x.device) if rounded else None
+    if T:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_branch_norm(x.data_ptr(), _p(a), float(ca), _p(b), float(cb), _p(sh), _p(sg), ldsg,
+                                                             _p(moe.y) if moe else None, _p(moe.place_of) if moe else None, _p(moe.wts) if moe else None,
+                                                             moe.wts.shape[1] if moe else 0, None, T, W, w.data_ptr(), 1 if center else 0, float(eps), _p(h),
+                                                             act_code(w.dtype), _stream()), "hy_branch_norm")
+    return h
+
+
+def norm_rows(x: torch.Tensor, rows: torch.Tensor, w: torch.Tensor, eps: float, *, center: bool = True) -> torch.Tensor:
+    """N(x[rows]) * w in w's dtype for the fp32 stream x (layer norm with `center`, else RMS norm); x is left as it is."""
+    _dev(x, torch.float32, "norm_rows.x"); _dev(rows, torch.int32, "norm_rows.rows")
+    W = x.shape[1]
+    if not x.is_contiguous() or w.numel() != W or not w.is_contiguous():
+        raise _C.Mi355Error(f"norm_rows: stream {tuple(x.shape)} (contiguous) against a weight {tuple(w.shape)}")
+    n = rows.numel()
+    h = torch.empty(n, W, dtype=w.dtype, device=x.device)
+    if n:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_branch_norm(x.data_ptr(), None, 1.0, None, 1.0, None, None, 0, None, None, None, 0, rows.data_ptr(), n, W,
+                                                             w.data_ptr(), 1 if center else 0, float(eps), h.data_ptr(), act_code(w.dtype), _stream()),
+                        "hy_norm_rows")
+    return h
+
+
 def depth_mix_norm(x: torch.Tensor, a: Optional[torch.Tensor], stack: torch.Tensor, n: int, coef: torch.Tensor, w1: Optional[torch.Tensor], eps: float, *,
                    weight_offset: float = 0.0, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """The end of layer n - 1 of a stack whose layers read a weighted average of ALL earlier results: stack[n] <- x + a (the layer's own result; a may
@@ -145,10 +211,12 @@ def depth_mix_norm(x: torch.Tensor, a: Optional[torch.Tensor], stack: torch.Tens
 
 class MoeSum:
     """A mixture's weighted sum still to be formed: sum_k wts[t, k] * y[place_of[t, k]] (+ extra[t]).  residual_norm takes it as a branch and
-    forms it while it updates the stream; moe_combine forms it on its own."""
+    forms it while it updates the stream; moe_combine forms it on its own.  extra_gate (fp32 [T], any stride): extra[t] is multiplied by
+    sigmoid(extra_gate[t]) (branch_norm forms that)."""
 
-    def __init__(self, y: torch.Tensor, place_of: torch.Tensor, wts: torch.Tensor, extra: Optional[torch.Tensor] = None):
-        self.y, self.place_of, self.wts, self.extra = y, place_of, wts, extra
+    def __init__(self, y: torch.Tensor, place_of: torch.Tensor, wts: torch.Tensor, extra: Optional[torch.Tensor] = None,
+                 extra_gate: Optional[torch.Tensor] = None):
+        self.y, self.place_of, self.wts, self.extra, self.extra_gate = y, place_of, wts, extra, extra_gate
 
 
 def residual_norm(x: torch.Tensor, a: Optional[torch.Tensor], b, mult: float, w1: torch.Tensor,
@@ -198,10 +266,11 @@ def attn_geometry(heads, kv_heads, dim, vdim, rot_dims, rot_layout, v_layout, pa
 
 def attn_prep(qkv: torch.Tensor, koff: int, voff: int, geom, kfreq, vfreq, v_norm: bool, eps: float, pos, seq, block_table,
               kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], *, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
-              mag: float = 1.0, q_temp=None, cache_dtype: Optional[torch.dtype] = None):
+              mag: float = 1.0, q_temp=None, cache_dtype: Optional[torch.dtype] = None, norm_whole: bool = False):
     """Rotate the query heads of qkv (fp32 [T, ld], in place); with caches: rotate the keys, unit-norm and rotate the values, and write both
     to their pages.  q_norm / k_norm ([dim] in the cache dtype): queries / keys are brought to unit RMS per head and multiplied by the weight
-    before the rotation; mag multiplies cos and sin; q_temp = (coef, every): queries are multiplied by 1 + coef ln(floor((p + 1) / every) + 1)."""
+    before the rotation; mag multiplies cos and sin; q_temp = (coef, every): queries are multiplied by 1 + coef ln(floor((p + 1) / every) + 1).
+    norm_whole: q_norm is [heads * dim] and k_norm [kv_heads * dim], and the unit RMS is taken over all heads of the row at once."""
     _dev(qkv, torch.float32, "attn_prep.qkv")
     ld = _rows(qkv, "attn_prep.qkv")
     T = qkv.shape[0]
@@ -211,12 +280,13 @@ def attn_prep(qkv: torch.Tensor, koff: int, voff: int, geom, kfreq, vfreq, v_nor
     for t, nm in ((q_norm, "q_norm"), (k_norm, "k_norm")):
         if t is not None:
             _dev(t, dt, "attn_prep." + nm)
-            if t.numel() != geom[2] or not t.is_contiguous():
-                raise _C.Mi355Error(f"attn_prep.{nm}: {tuple(t.shape)} for heads of {geom[2]}")
+            want = geom[2] * ((geom[0] if nm == "q_norm" else geom[1]) if norm_whole else 1)
+            if t.numel() != want or not t.is_contiguous():
+                raise _C.Mi355Error(f"attn_prep.{nm}: {tuple(t.shape)} for {want} channels")
     coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp else (0.0, 1)
-    _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_prep_ex(qkv.data_ptr(), ld, koff, voff, geom, _p(kfreq), _p(vfreq), 1 if v_norm else 0, float(eps),
-                                                          pos.data_ptr(), seq.data_ptr(), _p(block_table), T, _p(kcache), _p(vcache), _p(q_norm), _p(k_norm),
-                                                          float(mag), coef, every, act_code(dt), _stream()), "hy_attn_prep")
+    _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_prep_ex2(qkv.data_ptr(), ld, koff, voff, geom, _p(kfreq), _p(vfreq), 1 if v_norm else 0, float(eps),
+                                                           pos.data_ptr(), seq.data_ptr(), _p(block_table), T, _p(kcache), _p(vcache), _p(q_norm), _p(k_norm),
+                                                           1 if norm_whole else 0, float(mag), coef, every, act_code(dt), _stream()), "hy_attn_prep")
 
 
 def _sink(sink: Optional[torch.Tensor], heads: int):
@@ -345,7 +415,7 @@ def head_norm(o: torch.Tensor, heads: int, vdim: int, w: Optional[torch.Tensor],
 
 def dense_grouped(x: torch.Tensor, w: torch.Tensor, *, x_step: int = 0, y_step: int = 0, offs: Optional[torch.Tensor] = None,
                   gather: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None, rows: Optional[int] = None, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
-                  act: int = ACT_NONE, out: Optional[torch.Tensor] = None, mul_sigmoid: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  act: int = ACT_NONE, out: Optional[torch.Tensor] = None, mul_sigmoid: Optional[torch.Tensor] = None, act_param: float = 0.0) -> torch.Tensor:
     """One launch of G = w.shape[0] linears with the weights w [G, N, K].  mul_sigmoid: fp32 [M, width of the output] pre-activations (a column
     slice of a wider buffer is fine); every output is multiplied by the sigmoid of its entry before it is stored.
     Without offs every group takes all rows of x, reads its K inputs from column g * x_step and writes its outputs from column g * y_step
@@ -385,10 +455,10 @@ def dense_grouped(x: torch.Tensor, w: torch.Tensor, *, x_step: int = 0, y_step: 
         if mul_sigmoid.shape != (M, width):
             raise _C.Mi355Error(f"dense_grouped: gate {tuple(mul_sigmoid.shape)} for outputs [{M}, {width}]")
     if M:
-        _C.check_hybrid(_C.hybrid_lib().mi355_dense_grouped(x.data_ptr(), ldx, M, w.data_ptr(), N, K, None, out.data_ptr(), _rows(out, "dense_grouped.out"),
-                                                            1 if od == torch.float32 else 0, 1 if gated else 0, act, act_code(w.dtype), G, x_step, y_step,
-                                                            _p(offs), _p(gather), _p(tiles), 0 if tiles is None else (tiles.numel() - 1) // 2, _p(mul_sigmoid), ldg, 0,
-                                                            _stream()),
+        _C.check_hybrid(_C.hybrid_lib().mi355_dense_grouped_ex(x.data_ptr(), ldx, M, w.data_ptr(), N, K, None, out.data_ptr(), _rows(out, "dense_grouped.out"),
+                                                               1 if od == torch.float32 else 0, 1 if gated else 0, act, float(act_param), act_code(w.dtype), G, x_step,
+                                                               y_step, _p(offs), _p(gather), _p(tiles), 0 if tiles is None else (tiles.numel() - 1) // 2,
+                                                               _p(mul_sigmoid), ldg, 0, _stream()),
                         "dense_grouped")
     return out
 
@@ -441,16 +511,17 @@ def polynorm(z: torch.Tensor, coef, eps: float, dtype: torch.dtype) -> torch.Ten
     return out
 
 
-def moe_route(z: torch.Tensor, groups: int, keep: int, top: int):
-    """Router logits fp32 [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]): softmax scores, only experts of the `keep` best of
-    `groups` runs of neighbouring experts (a run scores as its best member) are eligible, the `top` best eligible are chosen."""
+def moe_route(z: torch.Tensor, groups: int, keep: int, top: int, *, sigmoid: bool = False, group_top: int = 1, scale: float = 1.0):
+    """Router logits fp32 [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]): softmax scores (sigmoid: a sigmoid of every logit), only
+    experts of the `keep` best of `groups` runs of neighbouring experts (a run scores as its best member, or with group_top = 2 as the sum of its
+    two best) are eligible, the `top` best eligible are chosen; their weights are score * scale."""
     _dev(z, torch.float32, "moe_route.z")
     T, E = z.shape
     ids = torch.empty(T, top, dtype=torch.int32, device=z.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=z.device)
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_route(z.data_ptr(), _rows(z, "moe_route.z"), T, E, groups, keep, top, ids.data_ptr(), wts.data_ptr(),
-                                                           _stream()), "hy_moe_route")
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_route_ex(z.data_ptr(), _rows(z, "moe_route.z"), T, E, groups, keep, top, ids.data_ptr(), wts.data_ptr(),
+                                                              1 if sigmoid else 0, int(group_top), float(scale), _stream()), "hy_moe_route")
     return ids, wts
 
 
@@ -470,21 +541,22 @@ def moe_align(ids: torch.Tensor, experts: int):
     return offs, src, place, tiles
 
 
-def moe_route_sorted(z: torch.Tensor, experts: int, groups: int, keep: int, top: int):
+def moe_route_sorted(z: torch.Tensor, experts: int, groups: int, keep: int, top: int, *, sigmoid: bool = False, group_top: int = 1, scale: float = 1.0):
     """moe_route followed by moe_align -> (ids, wts, offs, src_row, place_of, tiles); a few tokens (a decode step) take one launch for both."""
     _dev(z, torch.float32, "moe_route_sorted.z")
     T = z.shape[0]
     if z.shape[1] != experts:
         raise _C.Mi355Error(f"moe_route_sorted: logits {tuple(z.shape)} for {experts} experts")
     if not 0 < T <= 64 or 16 * (experts + groups) * 4 + experts * 8 > 48 * 1024:
-        ids, wts = moe_route(z, groups, keep, top)
+        ids, wts = moe_route(z, groups, keep, top, sigmoid=sigmoid, group_top=group_top, scale=scale)
         return (ids, wts) + moe_align(ids, experts)
     dev = z.device
     ids, wts = torch.empty(T, top, dtype=torch.int32, device=dev), torch.empty(T, top, dtype=torch.float32, device=dev)
     offs, src, place = torch.empty(experts + 1, dtype=torch.int32, device=dev), torch.empty(T * top, dtype=torch.int32, device=dev), torch.empty(T * top, dtype=torch.int32, device=dev)
     tiles = torch.empty(1 + 2 * (T * top // 64 + experts), dtype=torch.int32, device=dev)
-    _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_route_align(z.data_ptr(), _rows(z, "moe_route_sorted.z"), T, experts, groups, keep, top, ids.data_ptr(), wts.data_ptr(),
-                                                             offs.data_ptr(), src.data_ptr(), place.data_ptr(), tiles.data_ptr(), _stream()), "hy_moe_route_align")
+    _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_route_align_ex(z.data_ptr(), _rows(z, "moe_route_sorted.z"), T, experts, groups, keep, top, ids.data_ptr(),
+                                                                wts.data_ptr(), offs.data_ptr(), src.data_ptr(), place.data_ptr(), tiles.data_ptr(),
+                                                                1 if sigmoid else 0, int(group_top), float(scale), _stream()), "hy_moe_route_align")
     return ids, wts, offs, src, place, tiles
 
 

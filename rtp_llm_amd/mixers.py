@@ -20,8 +20,11 @@
     up-projection is moved to the query side and the value up-projection behind the weighted sum, so the paged kernels see multi-query
     attention over the cached rows.  Rotary with optional YaRN frequency scaling, a learned per-head softmax sink, a sigmoid output gate.
   * ``Retention`` -- the same recurrence with one constant decay per head, rotated q and k, unit-RMS heads and a silu output gate.
+  * ``LightningAttention`` -- that recurrence with silu on q, k and v, one RMS norm over all heads together and a sigmoid output gate.
+  * ``ParallelMixer`` -- two of the mixers side by side on one input, their outputs added with a constant each.
   * ``GatedMLP``, ``PolyNormMLP``, ``RoutedExperts`` -- feed-forward branches: gated dense, dense with the PolyNorm activation, and a
-    mixture of gated experts (softmax router, group-limited top-k, optional shared expert) over one grouped linear per projection.
+    mixture of gated experts (softmax or sigmoid router, group-limited top-k, optional shared expert with an optional gate of its own) over
+    one grouped linear per projection.  The gated activations include the clamped form min(g, L) sigmoid(1.702 min(g, L)) (clamp(u) + 1).
 
 All take the normed activations of a ragged batch (``StepBatch``) and return the fp32 branch output [T, width]."""
 import math
@@ -44,19 +47,38 @@ class RotaryScaling:
 
 
 @dataclass
+class WavelengthScaling:
+    """Scaling by wavelength (the Llama 3.1 rule): with l = 2 pi / step, steps with l < original / high stay, steps with l > original / low are divided
+    by `factor`, and between the two the step is (1 - s) step / factor + s step with s = (original / l - low) / (high - low).  cos and sin keep
+    their magnitude."""
+    factor: float
+    original: float
+    low: float
+    high: float
+
+
+@dataclass
 class RotarySpec:
     dims: int
     base: float
     layout: str = "interleaved"          # "interleaved": pairs (2i, 2i+1); "halves": (i, i + dims / 2)
-    scaling: Optional[RotaryScaling] = None
+    scaling: Optional[object] = None     # RotaryScaling (YaRN) | WavelengthScaling | None
 
     @staticmethod
-    def from_json(rot: Optional[dict], layout: str) -> Optional["RotarySpec"]:
+    def from_json(rot: Optional[dict], layout: str, scaling: str = "yarn") -> Optional["RotarySpec"]:
+        """scaling: how rot.scaling is read: "yarn" {factor, original, fast, slow} or "wavelength" {factor, original, low, high}."""
         if not rot or not int(rot.get("dims", 0)):
             return None
         sc = rot.get("scaling")
-        return RotarySpec(int(rot["dims"]), float(rot["base"]), layout,
-                          RotaryScaling(float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"])) if sc else None)
+        if not sc:
+            spec = None
+        elif scaling == "yarn":
+            spec = RotaryScaling(float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"]))
+        elif scaling == "wavelength":
+            spec = WavelengthScaling(float(sc["factor"]), float(sc["original"]), float(sc["low"]), float(sc["high"]))
+        else:
+            raise ValueError(f"rotary scaling {scaling!r}")
+        return RotarySpec(int(rot["dims"]), float(rot["base"]), layout, spec)
 
 
 @dataclass
@@ -80,6 +102,8 @@ class AttentionSpec:
     bias: bool = False                   # the q, k, v projections have biases
     out_bias: bool = False               # the output projection has a bias
     out_gate: bool = False               # head h's output is multiplied by sigmoid(W_g x)_h, one number per head
+    learned_sink: bool = False           # with sink: head h's sink logit is the checkpoint's `sink`[h] instead of 0
+    qk_norm_whole: bool = False          # with qk_norm: ONE RMS norm over all query heads (and one over all key heads) under weights [heads * dim]
 
 
 @dataclass
@@ -124,7 +148,14 @@ def rotary_table(rot: RotarySpec, device):
     i = torch.arange(rot.dims // 2, dtype=torch.float64)
     f = torch.pow(torch.tensor(float(rot.base), dtype=torch.float64), -2.0 * i / rot.dims)
     mag, sc = 1.0, rot.scaling
-    if sc is not None:
+    if isinstance(sc, WavelengthScaling):
+        if sc.high <= sc.low or sc.factor <= 0:
+            raise ValueError(f"rotary scaling: low {sc.low} high {sc.high} factor {sc.factor}")
+        lam = 2.0 * math.pi / f
+        blend = (sc.original / lam - sc.low) / (sc.high - sc.low)
+        mid = (1.0 - blend) * f / sc.factor + blend * f
+        f = torch.where(lam < sc.original / sc.high, f, torch.where(lam > sc.original / sc.low, f / sc.factor, mid))
+    elif sc is not None:
         at = lambda turns: rot.dims * math.log(sc.original / (2.0 * math.pi * turns)) / (2.0 * math.log(rot.base))
         lo, hi = max(math.floor(at(sc.fast)), 0), min(math.ceil(at(sc.slow)), rot.dims - 1)
         ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
@@ -140,8 +171,9 @@ def rotary_steps(n_pairs: int, span: int, base: float, device) -> torch.Tensor:
 
 
 class PagedChunkAttention:
-    """weights: q [H dim, W], k [G dim, W], v [G vdim, W] (absent with kv_from), o [W, H vdim]; by option q.b / k.b / v.b / o.b, q.norm / k.norm [dim],
-    g [H, W].  Every projection of the input (q | k | v | gate) is one linear."""
+    """weights: q [H dim, W], k [G dim, W], v [G vdim, W] (absent with kv_from), o [W, H vdim]; by option q.b / k.b / v.b / o.b, q.norm / k.norm [dim]
+    (or [H dim] / [G dim] when the norm runs over all heads at once), g [H, W], sink [H].  Every projection of the input (q | k | v | gate) is one
+    linear."""
 
     def __init__(self, spec: AttentionSpec, weights: Dict[str, torch.Tensor], eps: float, page: int, device):
         s = self.spec = spec
@@ -169,7 +201,17 @@ class PagedChunkAttention:
         self.vfreq = rotary_steps(s.vdim // 2, s.vdim, rot.base, device) if s.value_rot and rot else None
         self._geom = None
         self.use_tiles = True
-        self.sink = torch.zeros(s.heads, dtype=torch.float32, device=device) if s.sink else None
+        self.sink = None
+        if s.sink:
+            self.sink = weights["sink"].to(torch.float32).contiguous() if s.learned_sink else torch.zeros(s.heads, dtype=torch.float32, device=device)
+            if self.sink.numel() != s.heads:
+                raise ValueError(f"attention: {self.sink.numel()} sink logits for {s.heads} heads")
+        for t, n in ((self.q_norm, s.heads), (self.k_norm, s.kv_heads)):
+            if t is not None and t.numel() != s.dim * (n if s.qk_norm_whole else 1):
+                raise ValueError(f"attention: norm weight of {t.numel()} channels for {n} heads of {s.dim} ({'all heads at once' if s.qk_norm_whole else 'per head'})")
+
+    def cache_kind(self):
+        return "kv" if self.owns_cache else "kv_from"
 
     def cache_shapes(self):
         """(K page tensor shape, V page tensor shape) without the leading page count."""
@@ -186,14 +228,17 @@ class PagedChunkAttention:
                                                   num_pages))
         return self._geom[1]
 
-    def forward(self, h: torch.Tensor, batch: StepBatch, kcache: torch.Tensor, vcache: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, batch: StepBatch, kcache: torch.Tensor, vcache: torch.Tensor, proj: Optional[torch.Tensor] = None,
+                out_proj: bool = True) -> torch.Tensor:
+        """proj: h w_in^T (+ b_in) in fp32 when the caller has computed it (as columns of a linear shared with other projections of h; the query
+        columns are turned in place).  out_proj False: the heads' outputs [T, H vdim] come back without the output projection."""
         s = self.spec
         geom = self.geometry(batch.block_table.shape[1], kcache.shape[0])
-        qkv = hops.dense_linear(h, self.w_in, self.b_in, out_dtype=torch.float32)
+        qkv = hops.dense_linear(h, self.w_in, self.b_in, out_dtype=torch.float32) if proj is None else proj
         write = self.owns_cache
         hops.attn_prep(qkv, self.koff, self.voff, geom, self.kfreq, self.vfreq, s.value_norm, self.eps, batch.pos, batch.seq, batch.block_table,
                        kcache if write else None, vcache if write else None, q_norm=self.q_norm, k_norm=self.k_norm, mag=self.mag, q_temp=s.q_temp,
-                       cache_dtype=kcache.dtype)
+                       cache_dtype=kcache.dtype, norm_whole=s.qk_norm_whole)
         T = qkv.shape[0]
         extra = dict(window=s.window, softcap=s.softcap, out_gate=qkv[:, self.goff:self.goff + s.heads] if s.out_gate else None)
         # prompt portions (tiles mostly full) go to the matrix-core kernel, decode rows to the one that spreads a row's keys over four waves
@@ -204,7 +249,7 @@ class PagedChunkAttention:
         else:
             o = hops.attn_rows(qkv, s.scale, geom, s.chunk, self.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, kcache, vcache, s.heads, s.vdim,
                                **extra)
-        return hops.dense_linear(o, self.w_o, self.b_o, out_dtype=torch.float32)
+        return hops.dense_linear(o, self.w_o, self.b_o, out_dtype=torch.float32) if out_proj else o
 
 
 class GeneralizedDeltaRule:
@@ -396,6 +441,91 @@ class Retention:
         return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
 
 
+@dataclass
+class LightningSpec:
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple                         # one constant decay per head
+
+
+class LightningAttention:
+    """weights: q, k [H dim, W], v, g [H vdim, W], norm [H vdim], o [W, H vdim].  Linear attention with a constant decay per head:
+    S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with q, k, v = silu of their projections and the state in an fp32 slot.  The heads TOGETHER
+    are brought to unit RMS under `norm`, multiplied by sigmoid(W_g h) and projected."""
+
+    def __init__(self, spec: LightningSpec, weights: Dict[str, torch.Tensor], eps: float, device):
+        s = self.spec = spec
+        self.eps = eps
+        if len(s.decay) != s.heads:
+            raise ValueError(f"lightning attention: {len(s.decay)} decays for {s.heads} heads")
+        hd, hv = s.heads * s.dim, s.heads * s.vdim
+        for n, rows in (("q", hd), ("k", hd), ("v", hv), ("g", hv)):
+            if weights[n].shape[0] != rows:
+                raise ValueError(f"lightning attention: weight {n} {tuple(weights[n].shape)} for {s.heads} heads of {s.dim} x {s.vdim}")
+        self.w_in = torch.cat([weights["q"], weights["k"], weights["v"], weights["g"]], 0).contiguous()
+        self.b_in = None
+        self.qo, self.ko, self.vo, self.go = 0, hd, 2 * hd, 2 * hd + hv
+        self.decay = torch.tensor([float(a) for a in s.decay], dtype=torch.float32, device=device)
+        self.norm = weights["norm"].contiguous()
+        if self.norm.numel() != hv:
+            raise ValueError(f"lightning attention: norm weight of {self.norm.numel()} channels for {hv}")
+        self.w_o = weights["o"].contiguous()
+        self.act = self.w_o.dtype
+
+    def cache_kind(self):
+        return "state"
+
+    def state_shape(self):
+        s = self.spec
+        return (s.heads, s.dim, s.vdim)
+
+    def forward(self, h: torch.Tensor, batch: StepBatch, state: torch.Tensor, proj: Optional[torch.Tensor] = None, out_proj: bool = True) -> torch.Tensor:
+        """proj: h w_in^T in fp32 when the caller has computed it.  out_proj False: the normed, gated heads [T, H vdim] come back unprojected."""
+        s = self.spec
+        if proj is None:
+            proj = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
+        o = hops.scan(hops.SCAN_FIXED_SILU, proj, self.qo, self.ko, self.vo, None, self.decay, None, 1.0, 1.0, s.heads, s.dim, s.vdim,
+                      batch.row_start, batch.slot, batch.first_pos, state, self.act)
+        o = hops.head_norm(o, 1, s.heads * s.vdim, self.norm, self.eps, proj, self.go, gate_act="sigmoid")
+        return hops.dense_linear(o, self.w_o, out_dtype=torch.float32) if out_proj else o
+
+
+class ParallelMixer:
+    """Two mixers side by side on the same input: left_scale * left(h) + right_scale * right(h).  Each side is any mixer of this module whose
+    forward takes `proj` (its input projections as columns of a shared linear): all projections of h, of both sides, are ONE linear.  The
+    layer's cache is the sides' caches one after the other (pages for an attention side, a state slot for a recurrent side).  forward returns
+    the two sides' outputs with their scales, (left, left_scale, right, right_scale): the sum is formed by the kernel that ends the sublayer."""
+
+    def __init__(self, left, right, left_scale: float, right_scale: float):
+        self.left, self.right, self.left_scale, self.right_scale = left, right, float(left_scale), float(right_scale)
+        for m in (left, right):
+            if getattr(m, "w_in", None) is None or not hasattr(m, "cache_kind"):
+                raise ValueError(f"parallel mixer: {type(m).__name__} cannot run beside another mixer")
+        nl = left.w_in.shape[0]
+        self.n_left, self.off_right = nl, nl + (-nl) % 4                     # the right side's columns start 16-byte aligned
+        wl, wr = left.w_in, right.w_in
+        zrow = torch.zeros(self.off_right - nl, wl.shape[1], dtype=wl.dtype, device=wl.device)
+        self.w_in = torch.cat([wl, zrow, wr], 0).contiguous()
+        self.b_in = None
+        if left.b_in is not None or right.b_in is not None:
+            zb = lambda n: torch.zeros(n, dtype=wl.dtype, device=wl.device)
+            self.b_in = torch.cat([left.b_in if left.b_in is not None else zb(nl), zb(self.off_right - nl),
+                                   right.b_in if right.b_in is not None else zb(wr.shape[0])]).contiguous()
+        left.w_in = right.w_in = None                                            # live on as rows of the shared weight
+
+    def cache_parts(self):
+        """Per side: how many cache tensors its forward takes (2: key and value pages; 1: a state)."""
+        return [2 if m.cache_kind() in ("kv", "kv_from") else 1 for m in (self.left, self.right)]
+
+    def forward(self, h: torch.Tensor, batch: StepBatch, *cache):
+        nl_c, _ = self.cache_parts()
+        proj = hops.dense_linear(h, self.w_in, self.b_in, out_dtype=torch.float32)
+        a = self.left.forward(h, batch, *cache[:nl_c], proj=proj[:, :self.n_left])
+        b = self.right.forward(h, batch, *cache[nl_c:], proj=proj[:, self.off_right:])
+        return a, self.left_scale, b, self.right_scale
+
+
 class PolyNormMLP:
     """down(a N(z) + b N(z^2) + c N(z^3) + e), z = up h, N = unit RMS over a token's hidden channels; coef = the four numbers (a, b, c, e)."""
 
@@ -417,6 +547,9 @@ class RouterSpec:
     top: int
     groups: int = 1                      # experts form `groups` runs of neighbours ...
     keep: int = 1                        # ... and only those of the `keep` best runs can be chosen
+    score: str = "softmax"               # "softmax" over the logits | "sigmoid" of each logit
+    group_top: int = 1                   # a run scores as its best expert (1) or as the sum of its two best (2)
+    scale: float = 1.0                   # the chosen experts weigh score * scale
 
 
 class RoutedExperts:
@@ -424,13 +557,25 @@ class RoutedExperts:
     by their softmax scores (not renormalised), plus an optional shared expert that every token runs.  The (token, choice) pairs are sorted
     by expert on the device and each projection of all experts is one grouped linear; nothing returns to the host."""
 
-    def __init__(self, router: RouterSpec, w_router: torch.Tensor, gates, ups, downs, shared: Optional["GatedMLP"] = None, act: str = "silu"):
+    def __init__(self, router: RouterSpec, w_router: torch.Tensor, gates, ups, downs, shared: Optional["GatedMLP"] = None, act: str = "silu",
+                 act_param: float = 0.0, shared_gate: Optional[torch.Tensor] = None):
+        """act_param: the activation's parameter (the limit of "swiglu_clamp").  shared_gate [1, W]: the shared expert's output is multiplied by
+        sigmoid(shared_gate . h), one number per token; its row rides behind the router's in one linear."""
         r = self.router = router
+        if r.score not in ("softmax", "sigmoid") or r.group_top not in (1, 2):
+            raise ValueError(f"experts: router score {r.score!r}, groups ranked by their best {r.group_top}")
         if len(gates) != r.experts or w_router.shape[0] != r.experts:
             raise ValueError(f"experts: router of {w_router.shape[0]}, {len(gates)} experts, config says {r.experts}")
         if r.experts % r.groups or not 1 <= r.keep <= r.groups or not 1 <= r.top <= (r.experts // r.groups) * r.keep:
             raise ValueError(f"experts: {r.experts} experts in {r.groups} groups, keep {r.keep}, top {r.top}")
         self.w_router = w_router.contiguous()
+        self.n_router = r.experts
+        if shared_gate is not None:
+            if shared is None or shared_gate.numel() != w_router.shape[1]:
+                raise ValueError("experts: a gate for the shared expert needs that expert and one weight per input channel")
+            pad = torch.zeros((-(r.experts + 1)) % 4, w_router.shape[1], dtype=w_router.dtype, device=w_router.device)
+            self.w_router = torch.cat([w_router, shared_gate.reshape(1, -1), pad], 0).contiguous()
+        self.shared_gated = shared_gate is not None
         ff, K = gates[0].shape
         pad = (-ff) % 32
         gu, dn = [], []
@@ -441,19 +586,26 @@ class RoutedExperts:
                 d = torch.cat([d, torch.zeros(d.shape[0], pad, dtype=d.dtype, device=d.device)], 1)
             gu.append(hops.group_gate_up(g, u)); dn.append(d)
         self.w_gate_up, self.w_down = torch.stack(gu).contiguous(), torch.stack(dn).contiguous()
-        self.shared, self.act = shared, hops.ACTIVATIONS[act]
+        self.shared, self.act, self.act_param = shared, hops.ACTIVATIONS[act], float(act_param)
 
     def forward(self, h: torch.Tensor, logits: Optional[torch.Tensor] = None, defer: bool = False):
         """logits: the router's fp32 logits [T, experts] when the caller has computed them (in a linear shared with other projections of h).
-        defer: return the parts of the weighted sum (hybrid_ops.MoeSum) for a residual kernel that forms it, instead of the summed tensor."""
+        defer: return the parts of the weighted sum (hybrid_ops.MoeSum) for a residual kernel that forms it, instead of the summed tensor
+        (a gated shared expert is always left to that kernel)."""
         r = self.router
+        sgate = None
         if logits is None:
             logits = hops.dense_linear(h, self.w_router, out_dtype=torch.float32)
-        ids, wts, offs, src, place, tiles = hops.moe_route_sorted(logits, r.experts, r.groups, r.keep, r.top)
+            if self.shared_gated:
+                logits, sgate = logits[:, :self.n_router], logits[:, self.n_router]
+        ids, wts, offs, src, place, tiles = hops.moe_route_sorted(logits, r.experts, r.groups, r.keep, r.top, sigmoid=r.score == "sigmoid",
+                                                                  group_top=r.group_top, scale=r.scale)
         n = ids.numel()
-        a = hops.dense_grouped(h, self.w_gate_up, offs=offs, gather=src, tiles=tiles, rows=n, gated=True, act=self.act)
+        a = hops.dense_grouped(h, self.w_gate_up, offs=offs, gather=src, tiles=tiles, rows=n, gated=True, act=self.act, act_param=self.act_param)
         y = hops.dense_grouped(a, self.w_down, offs=offs, tiles=tiles, rows=n, out_dtype=torch.float32)
-        parts = hops.MoeSum(y, place, wts, self.shared.forward(h) if self.shared is not None else None)
+        parts = hops.MoeSum(y, place, wts, self.shared.forward(h) if self.shared is not None else None, sgate)
+        if self.shared_gated and not defer:
+            raise ValueError("experts: a gated shared expert joins the sum in the kernel that ends the sublayer (defer=True)")
         return parts if defer else hops.moe_combine(parts)
 
 
@@ -461,7 +613,7 @@ class GatedMLP:
     """down(act(gate h) * up h) with the gate and up weights grouped for the fused epilogue of the dense linear.  Channel counts that are
     not a multiple of 32 are padded with zero channels (zero gate and up rows, zero down columns)."""
 
-    def __init__(self, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, act: str = "relu"):
+    def __init__(self, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, act: str = "relu", act_param: float = 0.0):
         ff, K = gate.shape
         pad = (-ff) % 32
         if pad:
@@ -470,7 +622,7 @@ class GatedMLP:
             down = torch.cat([down, torch.zeros(down.shape[0], pad, dtype=down.dtype, device=down.device)], 1)
         self.w_gate_up = hops.group_gate_up(gate, up)
         self.w_down = down.contiguous()
-        self.act = hops.ACTIVATIONS[act]
+        self.act, self.act_param = hops.ACTIVATIONS[act], float(act_param)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return hops.dense_linear(hops.dense_linear(h, self.w_gate_up, gated=True, act=self.act), self.w_down, out_dtype=torch.float32)
+        return hops.dense_linear(hops.dense_linear(h, self.w_gate_up, gated=True, act=self.act, act_param=self.act_param), self.w_down, out_dtype=torch.float32)

@@ -43,7 +43,7 @@ def load_engine(path: str, dtype: torch.dtype = torch.bfloat16, device="cuda:0",
     return fn(path, dtype, device, **engine_args)
 
 
-@register("Nufalorn", "Pokepel", "Nepudra")
+@register("Nufalorn", "Pokepel", "Nepudra", "Nudorax")
 def _load_hybrid(path, dtype, device, *, max_tokens: int = 8192, max_seqs: int = 4, max_step_tokens: int = 2048, page: int = 64):
     from .hybrid import load_hybrid_checkpoint
     from .scheduler import ServingEngine
