@@ -214,8 +214,8 @@ def main():
     ap.add_argument("--hybrid", action="store_true", help="instead of the default workload: prefill / decode throughput and kernel rooflines of the hybrid "
                     "decoder family beside the Qwen2 engine at equal sizes (rtp_llm_amd/bench_hybrid.py); 1 GPU")
     ap.add_argument("--hybrid-sizes", default="", help="--hybrid: comma-separated subset of w1024,w2048,w4096")
-    ap.add_argument("--hybrid-design", default="nufalorn", choices=["nufalorn", "pokepel", "nepudra"], help="--hybrid: which member of the family is measured; pokepel and nepudra run "
-                    "beside the Nufalorn member at equal sizes")
+    ap.add_argument("--hybrid-design", default="nufalorn", choices=["nufalorn", "pokepel", "nepudra", "nudorax"], help="--hybrid: which member of the family is measured; pokepel and nepudra run "
+                    "beside the Nufalorn member at equal sizes, nudorax beside the Pokepel member")
     ap.add_argument("--hybrid-prompt", type=int, default=2048)
     ap.add_argument("--hybrid-batch", type=int, default=16)
     args = ap.parse_args()

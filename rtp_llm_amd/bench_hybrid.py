@@ -9,6 +9,11 @@ Nufalorn kernels against their rooflines.
 `--hybrid-design nepudra` does the same for the Nepudra member (delta-rule recurrence, capped causal and sliding-window attention with gated
 heads, bigram embedding, depth-averaged sequential layers).
 
+`--hybrid-design nudorax` measures the Nudorax member (windowed sink attention beside lightning attention in every layer, layer norms on the
+sublayers' outputs, sigmoid-routed clamped experts with a gated shared expert) beside the Pokepel member, the family's closest (routed experts
+with a shared expert, fixed-decay recurrence, sink attention), at equal width, depth, heads, expert sizes and vocabulary, and its kernels beside
+the like Pokepel kernels against their rooflines.
+
 Output: one JSON line {"hybrid_bench": {size: {"hybrid": {...}, "qwen2": {...}, "kernels": [...]}}} (with --hybrid-design pokepel:
 {"pokepel": {...}, "nufalorn": {...}, "kernels": [...]})."""
 import json
@@ -196,6 +201,49 @@ def nepudra_weights(cfg, dev, seed=0, rank=64):
     return w
 
 
+def nudorax_config(s, experts=16, top=4, groups=4, keep=2, window=1024):
+    """Width, depth, heads and vocabulary of `s`; every layer runs grouped-query attention over a sliding window (learned sinks, queries and keys
+    normed over all heads, wavelength-scaled rotary steps) beside lightning attention with the recurrent sizes of Pokepel's retention layers,
+    and a mixture of `experts` clamped gated experts of a quarter of the FFN width (`top` of them + one gated shared expert per token)."""
+    layers, hd = [], s["hd"]
+    fe = s["ff"] // 4 // 32 * 32
+    for i in range(s["layers"]):
+        left = {"heads": s["heads"], "kv_heads": s["kv"], "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": window},
+                "rot": {"base": 1e6, "dims": hd, "scaling": {"factor": 16.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+        right = {"heads": s["heads"], "dim": hd // 2, "vdim": hd, "decay": [1.0 - 2.0 ** -(5 + h % 8) for h in range(s["heads"])]}
+        mlp = {"kind": "moe", "expert": {"ff": fe, "limit": 7.0}, "shared": {"ff": fe, "limit": 7.0},
+               "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": groups, "keep": keep}}}
+        layers.append({"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}, "mlp": mlp})
+    return {"architecture": "Nudorax", "layers": layers, "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "embedding": {"scale": s["width"] ** 0.5},
+            "logit_softcap": 30.0}
+
+
+def nudorax_weights(cfg, dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    W = cfg["width"]
+    lin = lambda o, i: (torch.randn(o, i, device=dev, generator=g) * i ** -0.5).bfloat16()
+    vec = lambda n, k=0.1, off=0.0: (torch.randn(n, device=dev, generator=g) * k + off).bfloat16()
+    w = {"embed": (torch.randn(cfg["vocab"], W, device=dev, generator=g) * W ** -0.5).bfloat16(), "final.norm": vec(W, 0.1, 1.0)}
+    for i, L in enumerate(cfg["layers"]):
+        p, a, b, mlp = f"l{i}.", L["mixer"]["left"], L["mixer"]["right"], L["mlp"]
+        w[p + "norm1"], w[p + "norm2"] = vec(W, 0.1, 1.0), vec(W, 0.1, 1.0)
+        H, G, d, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+        q = p + "mix.left."
+        for n, (o, k) in {"q": (H * d, W), "k": (G * d, W), "v": (G * dv, W), "o": (W, H * dv)}.items():
+            w[q + n] = lin(o, k)
+        w[q + "q.norm"], w[q + "k.norm"], w[q + "sink"] = vec(H * d, 0.1, 1.0), vec(G * d, 0.1, 1.0), vec(H, 1.0)
+        H, d, dv = b["heads"], b["dim"], b["vdim"]
+        q = p + "mix.right."
+        for n, (o, k) in {"q": (H * d, W), "k": (H * d, W), "v": (H * dv, W), "g": (H * dv, W), "o": (W, H * dv)}.items():
+            w[q + n] = lin(o, k)
+        w[q + "norm"] = vec(H * dv, 0.1, 1.0)
+        w[p + "mlp.router"], w[p + "mlp.shared.sg"] = lin(mlp["router"]["experts"], W), lin(1, W)
+        for n in [f"e{j}" for j in range(mlp["router"]["experts"])] + ["shared"]:
+            f = mlp["expert"]["ff"]
+            w[p + f"mlp.{n}.gate"], w[p + f"mlp.{n}.up"], w[p + f"mlp.{n}.down"] = lin(f, W), lin(f, W), lin(W, f)
+    return w
+
+
 def timed(fn, reps=5, warm=2, graph=False):
     """Seconds per call.  graph: the calls are captured into one HIP graph and the replay is timed, so the figure is the kernels' own
     time and not the host's launch path (what a graph-replayed step pays)."""
@@ -230,7 +278,8 @@ def timed(fn, reps=5, warm=2, graph=False):
 def bench_hybrid_engine(s, dev, prompt, batch, steps, design="nufalorn"):
     from .hybrid import HybridConfig, HybridModel
     from .scheduler import ServingEngine
-    make_cfg, make_w = {"pokepel": (pokepel_config, pokepel_weights), "nepudra": (nepudra_config, nepudra_weights)}.get(design, (hybrid_config, hybrid_weights))
+    make_cfg, make_w = {"pokepel": (pokepel_config, pokepel_weights), "nepudra": (nepudra_config, nepudra_weights),
+                        "nudorax": (nudorax_config, nudorax_weights)}.get(design, (hybrid_config, hybrid_weights))
     cfg = make_cfg(s)
     model = HybridModel(HybridConfig.from_json(cfg), make_w(cfg, dev), torch.bfloat16, dev)
     eng = ServingEngine(model, max_tokens=batch * (prompt + 8 * (steps + 3) + 128), max_seqs=batch, max_step_tokens=1 << 20)
@@ -636,23 +685,165 @@ def kernel_table_nepudra(s, dev, prompt):
     return rows
 
 
+def kernel_table_nudorax(s, dev, prompt):
+    """Nudorax's kernels at this size beside the like kernels of the Pokepel member, against max(bytes / HBM, flops / peak of the unit)."""
+    from . import hybrid_ops as hops
+    rows = []
+    timed_k = lambda fn: timed(fn, reps=10, warm=2, graph=True)
+    g = torch.Generator(device=dev).manual_seed(3)
+    bf = lambda *sh: torch.randn(*sh, device=dev, generator=g).bfloat16()
+    f32 = lambda *sh: torch.randn(*sh, device=dev, generator=g)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    W, H, G, hd = s["width"], s["heads"], s["kv"], s["hd"]
+    cfg, pcfg = nudorax_config(s), pokepel_config(s)
+    moe = cfg["layers"][0]["mlp"]
+    lat = next(L["mixer"] for L in pcfg["layers"] if L["type"] == "latent_attention")
+    R, dr = lat["kv_rank"], lat["rot_dim"]
+    dpad = -(-(R + dr) // 32) * 32
+    fe, E, top, gr, lim = moe["expert"]["ff"], moe["router"]["experts"], moe["router"]["top"], moe["router"]["groups"], moe["expert"]["limit"]
+    window = cfg["layers"][0]["mixer"]["left"]["mask"]["size"]
+
+    def add(family, name, shape, t, nbytes, flops, peak):
+        roof = max(nbytes / HBM, flops / peak)
+        rows.append({"family": family, "kernel": name, "shape": shape, "us": round(t * 1e6, 1), "roofline_us": round(roof * 1e6, 2),
+                     "x_roofline": round(t / roof, 1)})
+
+    page = 64
+    nblk = (prompt + page - 1) // page + 1
+    bt = torch.arange(nblk, dtype=torch.int32, device=dev).reshape(1, nblk)
+    sink = f32(H)
+    # attention: grouped-query pages under a sliding window with learned sinks, against one cached latent row per token for all heads (causal)
+    geom = hops.attn_geometry(H, G, hd, hd, hd, 1, 0, page, nblk, nblk)
+    lgeo = hops.attn_geometry(H, 1, dpad, R, 0, 0, 0, page, nblk, nblk, v_ld=dpad)
+    kc, vc, lc = bf(nblk, G, page, hd), bf(nblk, G, page, hd), bf(nblk, 1, page, dpad)
+    for T_, name in ((prompt, "prefill"), (1, "decode")):
+        pos = torch.arange(T_, dtype=torch.int32, device=dev) if T_ > 1 else i32([prompt - 1])
+        seq = torch.zeros(T_, dtype=torch.int32, device=dev)
+        q, lq = f32(T_, H * hd), f32(T_, H * dpad)
+        kw = float(sum(min(int(p) + 1, window) for p in pos.tolist()))
+        kall = float(sum(int(p) + 1 for p in pos.tolist()))
+        byt = lambda keys: min(prompt, keys) * G * hd * 2 * 2 + T_ * H * hd * 6
+        if T_ > 1:
+            t0 = torch.arange(0, T_, 16, dtype=torch.int32, device=dev)
+            tn = torch.full_like(t0, 16)
+            t = timed_k(lambda: hops.attn_tiles(q, hd ** -0.5, geom, 0, sink, None, pos, seq, bt, t0, tn, kc, vc, H, hd, window=window))
+            add("nudorax", f"attn_tiles prefill (window {window}, learned sinks)", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t, byt(prompt), 4.0 * kw * H * hd, MFMA_BF16)
+            t = timed_k(lambda: hops.attn_tiles(lq, 0.07, lgeo, 0, sink, None, pos, seq, bt, t0, tn, lc, lc, H, R))
+            add("pokepel", "attn_tiles latent prefill (causal, learned sinks)", f"T={T_} H={H} row={dpad} rank={R} ctx={prompt}", t, prompt * dpad * 2 + T_ * H * (dpad * 4 + R * 2),
+                2.0 * kall * H * (dpad + R), MFMA_BF16)
+        else:
+            t = timed_k(lambda: hops.attn_rows(q, hd ** -0.5, geom, 0, sink, None, pos, seq, bt, kc, vc, H, hd, window=window))
+            add("nudorax", f"attn_rows decode (window {window}, learned sinks)", f"T=1 H={H} G={G} hd={hd} ctx={prompt}", t, byt(window), 4.0 * kw * H * hd, MFMA_BF16)
+            t = timed_k(lambda: hops.attn_rows(lq, 0.07, lgeo, 0, sink, None, pos, seq, bt, lc, lc, H, R))
+            add("pokepel", "attn_rows latent decode (learned sinks)", f"T=1 H={H} row={dpad} rank={R} ctx={prompt}", t, prompt * dpad * 2, 2.0 * kall * H * (dpad + R), MFMA_BF16)
+    # before the scores: norm over all heads + turn + page write, against latent norm + turn + page write + query split
+    freq = torch.ones(hd // 2, device=dev) * 1e-3
+    lgeom = hops.latent_geometry(H, hd, dr, R, dpad, dr, page, nblk, nblk)
+    for T_ in (prompt, 8):
+        pos, seq = torch.arange(T_, dtype=torch.int32, device=dev), torch.zeros(T_, dtype=torch.int32, device=dev)
+        qkv, qn_, kn_ = f32(T_, (H + 2 * G) * hd), bf(H * hd), bf(G * hd)
+        t = timed_k(lambda: hops.attn_prep(qkv, H * hd, (H + G) * hd, geom, freq, None, False, 1e-6, pos, seq, bt, kc, vc, q_norm=qn_, k_norm=kn_, norm_whole=True))
+        add("nudorax", "attn_prep (norm over all heads, turn, page write)", f"T={T_} H={H} G={G}", t, T_ * ((H + 2 * G) * hd * 4 + H * hd * 4 + 2 * G * hd * 2), 0, VALU_F32)
+        proj, qn, qabs, cw = f32(T_, H * (hd + dr) + R + dr), bf(T_, H * hd), f32(T_, H * dpad), bf(R)
+        t = timed_k(lambda: hops.latent_prep(proj, H * (hd + dr), lgeom, freq[: dr // 2], 1.2, cw, 1e-6, pos, seq, bt, qn, qabs, lc.view(nblk, page, dpad)))
+        add("pokepel", "latent_prep", f"T={T_} H={H}", t, T_ * (H * (hd + dr) * 4 + H * hd * 2 + H * (dpad - R) * 4 + dpad * 2), 0, VALU_F32)
+    # recurrence: fixed decay with silu on q, k, v inside the scan, against fixed decay after a separate turn of q and k; then the norm + gate
+    d = hd // 2
+    for T_, name in ((prompt, "prefill"), (8, "decode b=8")):
+        nseq = 1 if T_ > 8 else 8
+        proj = f32(T_, 2 * H * d + 2 * H * hd)
+        rs = torch.arange(0, T_ + 1, T_ // nseq, dtype=torch.int32, device=dev)
+        slot, fp = torch.arange(nseq, dtype=torch.int32, device=dev), torch.ones(nseq, dtype=torch.int32, device=dev)
+        state = torch.zeros(nseq, H, d, hd, device=dev)
+        decay = torch.full((H,), 0.97, device=dev)
+        nb, fl = T_ * (2 * H * d + 2 * H * hd) * 4 + 2 * nseq * H * d * hd * 4, 4.0 * T_ * H * d * hd
+        t = timed_k(lambda: hops.scan(hops.SCAN_FIXED_SILU, proj, 0, H * d, 2 * H * d, None, decay, None, 1.0, 1.0, H, d, hd, rs, slot, fp, state, torch.bfloat16))
+        add("nudorax", f"scan lightning (silu inside) {name}", f"T={T_} H={H} dim={d} vdim={hd}", t, nb, fl, VALU_F32)
+        t = timed_k(lambda: hops.scan(hops.SCAN_FIXED, proj, 0, H * d, 2 * H * d, None, decay, None, 1.0, 1.0, H, d, hd, rs, slot, fp, state, torch.bfloat16))
+        add("pokepel", f"scan retention {name}", f"T={T_} H={H} dim={d} vdim={hd}", t, nb, fl, VALU_F32)
+        o, wn = f32(T_, H * hd), bf(H * hd)
+        t = timed_k(lambda: hops.head_norm(o, 1, H * hd, wn, 1e-6, proj, 2 * H * d + H * hd, gate_act="sigmoid"))
+        add("nudorax", f"norm over all heads (weight, sigmoid gate) {name}", f"T={T_} H={H} vdim={hd}", t, T_ * H * hd * 10, 0, VALU_F32)
+        t = timed_k(lambda: hops.head_norm(o, H, hd, None, 1e-6, proj, 2 * H * d + H * hd, out_dtype=torch.bfloat16))
+        add("pokepel", f"norm per head (silu gate) {name}", f"T={T_} H={H} vdim={hd}", t, T_ * H * hd * 10, 0, VALU_F32)
+    # experts: routing + sorting, both grouped linears with the clamped gate, and the sublayer's end (mixture sum + gated shared expert + layer norm +
+    # residual + rounded copy) against Pokepel's (gated residual + mixture sum + RMS norm)
+    for T_ in (prompt, 8, 1):
+        h = bf(T_, W)
+        z = f32(T_, E + 4) * 2
+        t = timed_k(lambda: hops.moe_route_sorted(z[:, :E], E, gr["count"], gr["keep"], top, sigmoid=True, group_top=2, scale=2.5))
+        add("nudorax", "moe route + sort (sigmoid, groups by two best)", f"T={T_} E={E} top={top}", t, T_ * (E * 4 + top * 16), 0, VALU_F32)
+        t = timed_k(lambda: hops.moe_route_sorted(z[:, :E], E, gr["count"], gr["keep"], top))
+        add("pokepel", "moe route + sort (softmax, groups by best)", f"T={T_} E={E} top={top}", t, T_ * (E * 4 + top * 16), 0, VALU_F32)
+        ids, wts = hops.moe_route(z[:, :E], gr["count"], gr["keep"], top, sigmoid=True, group_top=2, scale=2.5)
+        offs, src, place, tiles = hops.moe_align(ids, E)
+        n = T_ * top
+        used = len(set(ids.flatten().tolist()))
+        wgu = torch.stack([hops.group_gate_up(bf(fe, W), bf(fe, W)) for _ in range(E)]).contiguous()
+        for fam, act, par in (("nudorax", hops.ACT_SWIGLU_CLAMP, lim), ("pokepel", hops.ACT_SILU, 0.0)):
+            t = timed_k(lambda: hops.dense_grouped(h, wgu, offs=offs, gather=src, tiles=tiles, rows=n, gated=True, act=act, act_param=par))
+            add(fam, "dense_grouped experts gated (%s)" % ("clamped" if par else "silu"), f"M={T_}x{top} E={E} ({used} used) N={2 * fe} K={W}", t,
+                used * 2 * fe * W * 2 + n * (W + fe) * 2, 2.0 * n * 2 * fe * W, MFMA_BF16)
+        y, extra = f32(n, W), f32(T_, W)
+        xs_, as_, gt_, w1_ = f32(T_, W), f32(T_, W), f32(T_, 2 * W), bf(W)
+        t = timed_k(lambda: hops.branch_norm(xs_, w1_, 1e-6, moe=hops.MoeSum(y, place, wts, extra, z[:, E]), rounded=True))
+        add("nudorax", "mixture sum + gated shared + layer norm + residual", f"T={T_} top={top} W={W}", t, (n + 3 * T_) * W * 4 + T_ * W * 2, 0, VALU_F32)
+        t = timed_k(lambda: hops.residual_norm(xs_, as_, hops.MoeSum(y, place, wts, extra), 1.0, w1_, None, 1e-6, gate=gt_))
+        add("pokepel", "gated residual + mixture sum + norm", f"T={T_} top={top} W={W}", t, (n + 7 * T_) * W * 4 + T_ * W * 2, 0, VALU_F32)
+    # the mixer sublayer's end (two weighted branches + layer norm + residual + rounded copy), the last norm on gathered rows, the embedding
+    for T_ in (prompt, 8):
+        x, a, b, gt = f32(T_, W), f32(T_, W), f32(T_, W), f32(T_, 2 * W)
+        w1 = bf(W)
+        t = timed_k(lambda: hops.branch_norm(x, w1, 1e-6, a=a, ca=1.5, b=b, cb=0.75, rounded=True))
+        add("nudorax", "two branches + layer norm + residual (fp32 stream)", f"M={T_} W={W}", t, stream_bytes(T_, W, 4, 1), 0, VALU_F32)
+        t = timed_k(lambda: hops.residual_norm(x, a, b, 1.0, w1, None, 1e-6, gate=gt))
+        add("pokepel", "gated residual + norm (fp32 stream)", f"M={T_} W={W}", t, stream_bytes(T_, W, 6, 1), 0, VALU_F32)
+        ids = torch.randint(0, s["vocab"], (T_,), device=dev, dtype=torch.int32)
+        table = bf(s["vocab"], W)
+        t = timed_k(lambda: hops.embed_scaled(ids, table, 8.0, rounded=True))
+        add("nudorax", "embedding x scale (stream + rounded copy)", f"M={T_} W={W}", t, T_ * W * (2 + 4 + 2), 0, VALU_F32)
+        t = timed_k(lambda: hops.embed(ids, table))
+        add("pokepel", "embedding", f"M={T_} W={W}", t, T_ * W * (2 + 4), 0, VALU_F32)
+    rows_ = torch.arange(8, dtype=torch.int32, device=dev)
+    x8, w1 = f32(8, W), bf(W)
+    t = timed_k(lambda: hops.norm_rows(x8, rows_, w1, 1e-6))
+    add("nudorax", "last layer norm on gathered rows", f"M=8 W={W}", t, 8 * W * 6, 0, VALU_F32)
+    t = timed_k(lambda: hops.residual_norm(x8, None, None, 1.0, w1, None, 1e-6, rows=rows_))
+    add("pokepel", "last norm on gathered rows", f"M=8 W={W}", t, 8 * W * 6, 0, VALU_F32)
+    # linears: ONE input linear per layer for both sides (left q | k | v, right q | k | v | g) against Pokepel's (mixer inputs | gates | router)
+    nl, nr = (H + 2 * G) * hd, 2 * H * d + 2 * H * hd
+    npk = H * (hd + dr) + R + dr + H * hd + 2 * W + E
+    for M_ in (prompt, 8, 1):
+        x = bf(M_, W)
+        for fam, N_ in (("nudorax", nl + nr), ("pokepel", npk // 4 * 4)):
+            wi = bf(N_, W)
+            t = timed_k(lambda: hops.dense_linear(x, wi, out_dtype=torch.float32))
+            add(fam, "dense_linear all projections of the input (fp32 out)", f"M={M_} N={N_} K={W}", t, N_ * W * 2 + M_ * (W * 2 + N_ * 4), 2.0 * M_ * N_ * W, MFMA_BF16)
+    return rows
+
+
 def stream_bytes(T_, W, f32_streams, bf16_streams):
     return T_ * W * (4 * f32_streams + 2 * bf16_streams)
 
 
+KERNEL_TABLES = {"pokepel": (kernel_table_pokepel, "nufalorn"), "nepudra": (kernel_table_nepudra, "nufalorn"), "nudorax": (kernel_table_nudorax, "pokepel")}
+
+
 def run_pokepel(args, dev, sizes, member="pokepel"):
+    """A member beside the member of the family that is closest to it (KERNEL_TABLES), engines and kernels."""
+    table, beside = KERNEL_TABLES[member]
     prompt, batch, steps = args.hybrid_prompt, args.hybrid_batch, args.steps
     out = {}
     for name in sizes:
         s = SIZES[name]
         log(f"[hybrid bench] {name}: {s}")
         rec = {"config": s, "prompt": prompt, "batch": batch}
-        for design in (member, "nufalorn"):
+        for design in (member, beside):
             rec[design], model, eng = bench_hybrid_engine(s, dev, prompt, batch, steps, design)
             del model, eng
             torch.cuda.empty_cache()
             log(f"[hybrid bench] {name} {design}: {rec[design]}")
-        rec["kernels"] = (kernel_table_pokepel if member == "pokepel" else kernel_table_nepudra)(s, dev, prompt)
+        rec["kernels"] = table(s, dev, prompt)
         for r in rec["kernels"]:
             log(f"    {r['family']:8s} {r['kernel']:64s} {r['shape']:48s} {r['us']:10.1f} us  roofline {r['roofline_us']:9.2f} us  x{r['x_roofline']}")
         out[name] = rec
@@ -666,7 +857,7 @@ def run(args):
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     sizes = [x for x in (args.hybrid_sizes.split(",") if args.hybrid_sizes else SIZES)]
-    if getattr(args, "hybrid_design", "nufalorn") in ("pokepel", "nepudra"):
+    if getattr(args, "hybrid_design", "nufalorn") in KERNEL_TABLES:
         return run_pokepel(args, dev, sizes, args.hybrid_design)
     prompt, batch, steps = args.hybrid_prompt, args.hybrid_batch, args.steps
     out = {}

@@ -197,43 +197,87 @@ __device__ __forceinline__ float hy_block_sum(float v, float* red) {       // re
 // Mean and variance are taken in two passes over the row kept in LDS; everything is fp32.
 struct BranchTerms { const float* a; float ca; const float* b; float cb; const float* sh; const float* sg; int ldsg; };
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void hy_branch_norm_kernel(float* x, BranchTerms bt, MoeSum ms, const int32_t* self_rows, const T* w, int center, float eps,
                                                              int W, T* h) {
     extern __shared__ __attribute__((aligned(16))) float hy_xs[];
     __shared__ float red[4];
+    constexpr int V = VEC ? 4 : 1, KMAX = 8;
     const int r = blockIdx.x, src = self_rows ? self_rows[r] : r;
     const size_t base = (size_t)src * W;
     const float gsh = (bt.sh && bt.sg) ? hy_sigmoid(bt.sg[(size_t)src * bt.ldsg]) : 1.f;
+    // the row's mixture weights and places, read once (the first KMAX choices; more are read in the loop)
+    float mw[KMAX];
+    const float* my[KMAX];
+    if (ms.y) {
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+            if (k < ms.top) { mw[k] = ms.wts[(size_t)src * ms.top + k]; my[k] = ms.y + (size_t)ms.place[(size_t)src * ms.top + k] * W; }
+    }
     float s1 = 0.f;
-    for (int c = threadIdx.x; c < W; c += 256) {
-        float y;
-        if (self_rows) y = x[base + c];
+    for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+        float y[4] = {0.f, 0.f, 0.f, 0.f}, t[4] = {0.f, 0.f, 0.f, 0.f};
+        if (self_rows) { if (VEC) hy_load4<float>(x + base + c, y); else y[0] = x[base + c]; }
         else {
-            y = 0.f;
-            if (bt.a) y = bt.ca * bt.a[base + c];
-            if (bt.b) y = __builtin_fmaf(bt.cb, bt.b[base + c], y);
-            if (ms.y) {                    // the chosen experts in choice order
-                float sum = 0.f;
-                for (int k = 0; k < ms.top; ++k)
-                    sum = __builtin_fmaf(ms.wts[(size_t)src * ms.top + k], ms.y[(size_t)ms.place[(size_t)src * ms.top + k] * W + c], sum);
-                y += sum;
+            if (bt.a) {
+                if (VEC) hy_load4<float>(bt.a + base + c, t); else t[0] = bt.a[base + c];
+#pragma unroll
+                for (int e = 0; e < V; ++e) y[e] = bt.ca * t[e];
             }
-            if (bt.sh) y = __builtin_fmaf(gsh, bt.sh[base + c], y);
+            if (bt.b) {
+                if (VEC) hy_load4<float>(bt.b + base + c, t); else t[0] = bt.b[base + c];
+#pragma unroll
+                for (int e = 0; e < V; ++e) y[e] = __builtin_fmaf(bt.cb, t[e], y[e]);
+            }
+            if (ms.y) {                    // the chosen experts in choice order
+                float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int k = 0; k < KMAX; ++k) {
+                    if (k >= ms.top) break;
+                    if (VEC) hy_load4<float>(my[k] + c, t); else t[0] = my[k][c];
+#pragma unroll
+                    for (int e = 0; e < V; ++e) sum[e] = __builtin_fmaf(mw[k], t[e], sum[e]);
+                }
+                for (int k = KMAX; k < ms.top; ++k) {
+                    const float wk = ms.wts[(size_t)src * ms.top + k];
+                    const float* yr = ms.y + (size_t)ms.place[(size_t)src * ms.top + k] * W + c;
+                    if (VEC) hy_load4<float>(yr, t); else t[0] = yr[0];
+#pragma unroll
+                    for (int e = 0; e < V; ++e) sum[e] = __builtin_fmaf(wk, t[e], sum[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < V; ++e) y[e] += sum[e];
+            }
+            if (bt.sh) {
+                if (VEC) hy_load4<float>(bt.sh + base + c, t); else t[0] = bt.sh[base + c];
+#pragma unroll
+                for (int e = 0; e < V; ++e) y[e] = __builtin_fmaf(gsh, t[e], y[e]);
+            }
         }
-        hy_xs[c] = y;
-        s1 += y;
+#pragma unroll
+        for (int e = 0; e < V; ++e) { hy_xs[c + e] = y[e]; s1 += y[e]; }
     }
     const float mean = center ? hy_block_sum(s1, red) / (float)W : 0.f;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < W; c += 256) { const float d = hy_xs[c] - mean; ss = __builtin_fmaf(d, d, ss); }
+    for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) { const float d = hy_xs[c + e] - mean; ss = __builtin_fmaf(d, d, ss); }
+    }
     const float inv = 1.f / sqrtf(hy_block_sum(ss, red) / (float)W + eps);
-    for (int c = threadIdx.x; c < W; c += 256) {
-        const float n = (hy_xs[c] - mean) * inv * (float)w[c];
-        if (self_rows) { h[(size_t)r * W + c] = (T)n; continue; }
-        const float v = x[base + c] + n;
-        x[base + c] = v;
-        if (h) h[base + c] = (T)v;
+    for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+        float g[4], n[4], v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (VEC) hy_load4<T>(w + c, g); else g[0] = (float)w[c];
+#pragma unroll
+        for (int e = 0; e < V; ++e) n[e] = (hy_xs[c + e] - mean) * inv * g[e];
+        if (self_rows) {
+            if (VEC) hy_store4<T>(h + (size_t)r * W + c, n); else h[(size_t)r * W + c] = (T)n[0];
+            continue;
+        }
+        if (VEC) hy_load4<float>(x + base + c, v); else v[0] = x[base + c];
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = v[e] + n[e];
+        if (VEC) hy_store4<float>(x + base + c, v); else x[base + c] = v[0];
+        if (h) { if (VEC) hy_store4<T>(h + base + c, v); else h[base + c] = (T)v[0]; }
     }
 }
 
@@ -1141,16 +1185,24 @@ __global__ __launch_bounds__(256) void hy_delta_kernel(DeltaParams p) {
 }
 
 // per-head RMS norm over vdim with a plain weight (null: none; shared by the heads, or w_heads: one per head and channel, [H * vdim]), optional
-// gate (silu, or gate_sigmoid: sigmoid): one wave per (row, head)
+// gate (silu, or gate_sigmoid: sigmoid): one block per (row, head), a single wave for heads of up to 256 channels and four waves beyond (one
+// "head" that spans all heads of a row: a norm over the whole concatenation)
 template <typename T>
-__global__ __launch_bounds__(64) void hy_head_norm_kernel(const float* o, int H, int vdim, const T* w, float eps, const float* gate, int ldg, int goff, T* out,
-                                                          int w_heads, int gate_sigmoid) {
-    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ __launch_bounds__(256) void hy_head_norm_kernel(const float* o, int H, int vdim, const T* w, float eps, const float* gate, int ldg, int goff, T* out,
+                                                           int w_heads, int gate_sigmoid) {
+    __shared__ float red[4];
+    const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, NT = blockDim.x;
     const float* src = o + ((size_t)r * H + h) * vdim;
     float ss = 0.f;
-    for (int c = lane; c < vdim; c += 64) ss = __builtin_fmaf(src[c], src[c], ss);
-    const float inv = 1.f / sqrtf(hy_wave_sum(ss) / (float)vdim + eps);
-    for (int c = lane; c < vdim; c += 64) {
+    for (int c = tid; c < vdim; c += NT) ss = __builtin_fmaf(src[c], src[c], ss);
+    ss = hy_wave_sum(ss);
+    if (NT > 64) {
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+        __syncthreads();
+        ss = (red[0] + red[1]) + (red[2] + red[3]);
+    }
+    const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
+    for (int c = tid; c < vdim; c += NT) {
         float v = src[c] * inv;
         if (w) v *= (float)w[w_heads ? h * vdim + c : c];
         if (gate) { const float gz = gate[(size_t)r * ldg + goff + h * vdim + c]; v *= gate_sigmoid ? hy_sigmoid(gz) : hy_silu(gz); }
@@ -1519,8 +1571,13 @@ extern "C" int mi355_hy_branch_norm(float* x, const float* a, float ca, const fl
     MI355_CHECK_ARG((size_t)W * 4 <= 64 * 1024, "hy_branch_norm: W=%d too wide for one block", W);
     const BranchTerms bt{a, ca, b, cb, sh, sg, ldsg};
     const MoeSum ms{moe_y, moe_place, moe_wts, moe_top};
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_branch_norm_kernel<T>, dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, bt, ms, self_rows, (const T*)w,
-                                              center, eps, W, (T*)h));
+    auto al = [](const void* p_) { return ((uintptr_t)p_ & 15) == 0; };
+    if (W % 4 == 0 && al(x) && al(a) && al(b) && al(sh) && al(moe_y) && al(w) && al(h))
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_branch_norm_kernel<T, true>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, bt, ms, self_rows,
+                                                  (const T*)w, center, eps, W, (T*)h));
+    else
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_branch_norm_kernel<T, false>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, bt, ms, self_rows,
+                                                  (const T*)w, center, eps, W, (T*)h));
     MI355_CHECK_LAUNCH("hy_branch_norm_kernel");
     return MI355_OK;
 }
@@ -1714,8 +1771,8 @@ extern "C" int mi355_hy_head_norm(const float* o, int32_t rows, int32_t H, int32
 extern "C" int mi355_hy_head_norm_ex(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
                                      int32_t goff, void* out, int32_t w_heads, int32_t gate_sigmoid, int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(o && out && rows > 0 && H > 0 && vdim > 0, "hy_head_norm: bad argument");
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_head_norm_kernel<T>, dim3(rows, H), dim3(64), 0, (hipStream_t)stream, o, H, vdim, (const T*)w, eps, gate, ldg,
-                                              goff, (T*)out, w_heads, gate_sigmoid));
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_head_norm_kernel<T>, dim3(rows, H), dim3(vdim > 256 ? 256 : 64), 0, (hipStream_t)stream, o, H, vdim, (const T*)w, eps,
+                                              gate, ldg, goff, (T*)out, w_heads, gate_sigmoid));
     MI355_CHECK_LAUNCH("hy_head_norm_kernel");
     return MI355_OK;
 }
