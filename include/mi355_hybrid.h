@@ -112,6 +112,13 @@ int mi355_hy_branch_norm(float* x, const float* a, float ca, const float* b, flo
                          const float* moe_y, const int32_t* moe_place, const float* moe_wts, int32_t moe_top, const int32_t* self_rows, int32_t n,
                          int32_t W, const void* w, int32_t center, float eps, void* h, int32_t act_dtype, mi355_stream_t stream);
 
+/* The chunked form of the fixed-decay recurrence (long prompt portions): a plan of chunks, mi355_hy_scan over the chunks from zero states, the prefix over a
+ * sequence's chunks, and mi355_hy_scan in mode 6 / 7 adding what the chunk-start states contribute. */
+int mi355_hy_chunk_plan(const int32_t* row_start, int32_t nseq, int32_t C, int32_t max_chunks, int32_t* cs, int32_t* sc, int32_t* ids, int32_t* zeros,
+                        int32_t* ones, mi355_stream_t stream);
+int mi355_hy_chunk_prefix(const int32_t* cs, const int32_t* sc, const int32_t* slot, const int32_t* first_pos, int32_t nseq, const float* decay, int32_t H,
+                          int32_t per_head, float* chunk_state, float* state, mi355_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

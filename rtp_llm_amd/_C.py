@@ -195,6 +195,8 @@ HYBRID_SIGNATURES = {
     "mi355_hy_moe_route_align_ex": (i32, [vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp, i32, i32, f32, vp]),
     "mi355_hy_attn_prep_ex2": (i32, [vp, i32, i32, i32, ip, vp, vp, i32, f32, vp, vp, vp, i32, vp, vp, vp, vp, i32, f32, f32, i32, i32, vp]),
     "mi355_hy_embed_scaled": (i32, [vp, i32, vp, i32, i32, f32, vp, vp, i32, vp]),
+    "mi355_hy_chunk_plan": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp]),
+    "mi355_hy_chunk_prefix": (i32, [vp, vp, vp, vp, i32, vp, i32, i32, vp, vp, vp]),
     "mi355_hy_branch_norm": (i32, [vp, vp, f32, vp, f32, vp, vp, i32, vp, vp, vp, i32, vp, i32, i32, vp, i32, f32, vp, i32, vp]),
 }
 

@@ -889,6 +889,52 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
     }   // pass
 }
 
+// decay^n for a constant decay in [0, 1] and n >= 0 (n = 0: 1, also for a decay of 0)
+__device__ __forceinline__ float hy_decay_pow(float a, int n) { return n == 0 ? 1.f : exp2f((float)n * log2f(a)); }
+
+// ------------------------------------------------------------------------------------------------ fixed-decay recurrence over long prompts: chunks
+// A recurrence with a constant decay per head, S_t = a S_(t-1) + k_t v_t^T, splits into chunks of C tokens that are walked side by side:
+//   1. every chunk is walked from a ZERO state (hy_scan_kernel over the chunks as if they were sequences): its outputs lack the part that comes
+//      from the state at its start, and what it leaves is its own contribution L_c = sum_j a^(n - 1 - j) k_j v_j^T;
+//   2. hy_chunk_prefix_kernel runs over a sequence's chunks in order: the state at the start of chunk c is S_c, S_(c+1) = a^(n_c) S_c + L_c; the
+//      S_c replace the L_c in the scratch buffer, the last one goes to the sequence's slot;
+//   3. hy_scan_kernel with `apply`: out_t += a^(t + 1) S_c^T q_t for token t of chunk c.
+// The sums are those of the token-by-token walk in another order (fp32 throughout).  The plan: chunk i covers rows cs[i] .. cs[i + 1] - 1 (unused
+// trailing chunks are empty), sequence s owns chunks sc[s] .. sc[s + 1] - 1.
+__global__ __launch_bounds__(256) void hy_chunk_plan_kernel(const int32_t* row_start, int nseq, int C, int max_chunks, int32_t* cs, int32_t* sc, int32_t* ids,
+                                                            int32_t* zeros, int32_t* ones) {
+    __shared__ int total;
+    if (threadIdx.x == 0) {
+        int a = 0;
+        for (int s_ = 0; s_ < nseq; ++s_) { sc[s_] = a; a += (row_start[s_ + 1] - row_start[s_] + C - 1) / C; }
+        sc[nseq] = a; total = a;
+    }
+    __syncthreads();
+    const int T = row_start[nseq];
+    for (int s_ = 0; s_ < nseq; ++s_) {
+        const int r0 = row_start[s_], c0 = sc[s_], n = sc[s_ + 1] - c0;
+        for (int i = threadIdx.x; i < n; i += 256) cs[c0 + i] = r0 + i * C;
+    }
+    for (int i = total + threadIdx.x; i <= max_chunks; i += 256) cs[i] = T;
+    for (int i = threadIdx.x; i < max_chunks; i += 256) { ids[i] = i; zeros[i] = 0; ones[i] = 1; }
+}
+
+__global__ __launch_bounds__(256) void hy_chunk_prefix_kernel(const int32_t* cs, const int32_t* sc, const int32_t* slot, const int32_t* first_pos, const float* decay,
+                                                              int H, int per_head, float* chunk_state, float* state) {
+    const int sq = blockIdx.x, h = blockIdx.y, e = blockIdx.z * 256 + threadIdx.x;
+    if (e >= per_head) return;
+    const float a = decay[h];
+    float* st = state + ((size_t)slot[sq] * H + h) * per_head + e;
+    float S = first_pos[sq] == 0 ? 0.f : *st;
+    for (int c = sc[sq]; c < sc[sq + 1]; ++c) {
+        float* cp = chunk_state + ((size_t)c * H + h) * per_head + e;
+        const float L = *cp;
+        *cp = S;
+        S = __builtin_fmaf(hy_decay_pow(a, cs[c + 1] - cs[c]), S, L);
+    }
+    *st = S;
+}
+
 // ------------------------------------------------------------------------------------------------ gated linear recurrence
 // Block = 64 value columns x DS groups of RD key rows: thread (c, ds) keeps S[ds * RD .. + RD - 1][c] in registers.  Tokens are staged `tok`
 // at a time: all threads compute the gates of the staged tokens once into LDS, then every thread walks the tokens in order (its RD rows:
@@ -906,6 +952,7 @@ struct ScanParams {
     float* state;                                   // [slots, H, dim, vdim]
     float* out;                                     // [rows, H * vdim]
     int tok;                                        // tokens staged per pass
+    int apply;                                      // fixed-decay modes: the state is only read: out[t] += decay^(t - first row + 1) * (S^T q_t), nothing is written back
 };
 
 template <typename T, int RD>
@@ -997,14 +1044,23 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
             const f32x4* kk = (const f32x4*)(k_s + t * dpad + ds * RD);
             const f32x4* aa = (const f32x4*)(a_s + t * dpad + ds * RD);
             float o[4] = {0.f, 0.f, 0.f, 0.f};
+            if (p.apply) {
 #pragma unroll
-            for (int j4 = 0; j4 < RD / 4; ++j4) {
-                const f32x4 a4 = aa[j4], k4 = kk[j4], q4 = qq[j4];
+                for (int j4 = 0; j4 < RD / 4; ++j4) {
+                    const f32x4 q4 = qq[j4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int j = j4 * 4 + e;
-                    s[j] = __builtin_fmaf(a4[e], s[j], k4[e] * vt);
-                    o[e] = __builtin_fmaf(s[j], q4[e], o[e]);
+                    for (int e = 0; e < 4; ++e) o[e] = __builtin_fmaf(s[j4 * 4 + e], q4[e], o[e]);
+                }
+            } else {
+#pragma unroll
+                for (int j4 = 0; j4 < RD / 4; ++j4) {
+                    const f32x4 a4 = aa[j4], k4 = kk[j4], q4 = qq[j4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int j = j4 * 4 + e;
+                        s[j] = __builtin_fmaf(a4[e], s[j], k4[e] * vt);
+                        o[e] = __builtin_fmaf(s[j], q4[e], o[e]);
+                    }
                 }
             }
             part_s[(t * DS + ds) * 64 + c] = (o[0] + o[1]) + (o[2] + o[3]);
@@ -1015,10 +1071,12 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
             if (v0 + cc >= p.vdim) continue;
             float o = 0.f;
             for (int k = 0; k < DS; ++k) o += part_s[(t * DS + k) * 64 + cc];
-            p.out[(size_t)(t0 + t) * p.H * p.vdim + h * p.vdim + v0 + cc] = o;
+            float* dst = p.out + (size_t)(t0 + t) * p.H * p.vdim + h * p.vdim + v0 + cc;
+            if (p.apply) *dst += o * hy_decay_pow(((const float*)p.lower)[h], t0 + t - r0 + 1);
+            else *dst = o;
         }
     }
-    if (vok) {
+    if (vok && !p.apply) {
 #pragma unroll
         for (int j = 0; j < RD; ++j) {
             const int d = ds * RD + j;
@@ -1714,6 +1772,7 @@ extern "C" int mi355_hy_attn_tiles_ex(const float* q, int32_t ldq, float scale, 
 // mode 1 (GLA):   q = proj q * qscale, k = proj k, a = sigmoid(z)^(1 / tau).
 // mode 2 (fixed): q = proj q, k = proj k, a = lower[h] (fp32 [H], one decay per head whatever act_dtype is).
 // mode 3 (fixed, silu): q = silu(proj q), k = silu(proj k), v = silu(proj v), a = lower[h] as in mode 2.
+// mode 6 / 7: modes 2 / 3 as the third pass of the chunked form: the states are only read, out[t] += a^(t - first row + 1) S^T q_t.
 // Sequence s owns rows row_start[s] .. row_start[s + 1] - 1 in order, continues the state in slot[s] (starts from zero when first_pos[s] == 0)
 // and leaves the new state there.  out fp32 [rows, H * vdim].
 extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_t qo, int32_t ko, int32_t vo, const float* z, int32_t ldz,
@@ -1721,21 +1780,46 @@ extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_
                              const int32_t* row_start, const int32_t* slot, const int32_t* first_pos, int32_t nseq, float* state, float* out,
                              int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(proj && row_start && slot && first_pos && state && out && nseq > 0 && H > 0 && dim > 0 && vdim > 0, "hy_scan: bad argument");
+    const int apply = mode & 4;                                   // mode + 4 (fixed-decay modes only): the read-only pass over chunk-start states
+    mode &= 3;
     MI355_CHECK_ARG(mode == SCAN_HGRN2 ? (lower && fbias) : (mode == SCAN_FIXED || mode == SCAN_FIXED_SILU) ? lower != nullptr : (mode == SCAN_GLA && z && tau > 0.f),
                     "hy_scan: mode %d lacks its gate inputs", mode);
+    MI355_CHECK_ARG(!apply || mode == SCAN_FIXED || mode == SCAN_FIXED_SILU, "hy_scan: the read-only pass belongs to the fixed-decay modes (mode %d)", mode);
+    mode |= apply;
     MI355_CHECK_ARG(dim <= 512, "hy_scan: key size %d > 512", dim);
     const int RD = dim <= 128 ? 8 : dim <= 256 ? 16 : 32;       // rows per thread: at most 16 groups of RD rows (1024 threads)
     const int DS = (dim + RD - 1) / RD;
     int tok = 16;                                                // staged tokens: keep the LDS buffers under 60 KiB
     auto lds_of = [&](int t) { return (size_t)(3 * t * DS * RD + t * 64 + t * DS * 64) * 4; };
     while (tok > 1 && lds_of(tok) > 60 * 1024) tok >>= 1;
-    ScanParams p{proj, ld, qo, ko, vo, z, ldz, lower, fbias, tau, qscale, mode, H, dim, vdim, row_start, slot, first_pos, state, out, tok};
+    ScanParams p{proj, ld, qo, ko, vo, z, ldz, lower, fbias, tau, qscale, mode & 3, H, dim, vdim, row_start, slot, first_pos, state, out, tok, (mode & 4) ? 1 : 0};
     const size_t lds = lds_of(tok);
     const dim3 grid(nseq, H, (vdim + 63) / 64);
     if (RD == 8)       HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_scan_kernel<T, 8>), grid, dim3(64 * DS), lds, (hipStream_t)stream, p));
     else if (RD == 16) HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_scan_kernel<T, 16>), grid, dim3(64 * DS), lds, (hipStream_t)stream, p));
     else               HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_scan_kernel<T, 32>), grid, dim3(64 * DS), lds, (hipStream_t)stream, p));
     MI355_CHECK_LAUNCH("hy_scan_kernel");
+    return MI355_OK;
+}
+
+// The plan of the chunked form for the sequences row_start[0 .. nseq]: chunks of C rows, at most max_chunks (>= rows / C + nseq).  cs int32 [max_chunks + 1],
+// sc int32 [nseq + 1]; ids / zeros / ones int32 [max_chunks]: 0, 1, 2 .. / all 0 / all 1 (slot and first_pos arrays of the chunk passes).
+extern "C" int mi355_hy_chunk_plan(const int32_t* row_start, int32_t nseq, int32_t C, int32_t max_chunks, int32_t* cs, int32_t* sc, int32_t* ids, int32_t* zeros,
+                                   int32_t* ones, mi355_stream_t stream) {
+    MI355_CHECK_ARG(row_start && cs && sc && ids && zeros && ones && nseq > 0 && C > 0 && max_chunks > 0, "hy_chunk_plan: nseq=%d C=%d chunks=%d", nseq, C, max_chunks);
+    hipLaunchKernelGGL(hy_chunk_plan_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, row_start, nseq, C, max_chunks, cs, sc, ids, zeros, ones);
+    MI355_CHECK_LAUNCH("hy_chunk_plan_kernel");
+    return MI355_OK;
+}
+
+// Pass 2 of the chunked form: chunk_state fp32 [chunks, H, dim * vdim] holds the chunks' own contributions and receives the states at their starts;
+// state [slots, H, dim * vdim] is continued (from zero where first_pos is 0) and receives the sequences' final states.  decay fp32 [H].
+extern "C" int mi355_hy_chunk_prefix(const int32_t* cs, const int32_t* sc, const int32_t* slot, const int32_t* first_pos, int32_t nseq, const float* decay, int32_t H,
+                                     int32_t per_head, float* chunk_state, float* state, mi355_stream_t stream) {
+    MI355_CHECK_ARG(cs && sc && slot && first_pos && decay && chunk_state && state && nseq > 0 && H > 0 && per_head > 0, "hy_chunk_prefix: nseq=%d H=%d", nseq, H);
+    hipLaunchKernelGGL(hy_chunk_prefix_kernel, dim3(nseq, H, (per_head + 255) / 256), dim3(256), 0, (hipStream_t)stream, cs, sc, slot, first_pos, decay, H, per_head,
+                       chunk_state, state);
+    MI355_CHECK_LAUNCH("hy_chunk_prefix_kernel");
     return MI355_OK;
 }
 

@@ -355,18 +355,69 @@ def attn_tiles(q: torch.Tensor, scale: float, geom, chunk: int, sink: Optional[t
     return out
 
 
+SCAN_CHUNK = 64            # tokens per chunk of the chunked form of the fixed-decay recurrence ...
+SCAN_CHUNKED_FROM = 256    # ... which steps of at least this many rows (and two or more rows per sequence on average) take
+SCAN_CHUNK_BYTES = 512 << 20
+
+
+class ChunkPlan:
+    """Chunks of a step's sequences for the chunked recurrence: device index arrays (see mi355_hy_chunk_plan) for one (row_start, chunk size)."""
+
+    def __init__(self, row_start: torch.Tensor, T: int, nseq: int, C: int):
+        self.C, self.max_chunks = C, T // C + nseq + 1
+        n = self.max_chunks
+        buf = torch.empty(4 * n + 1 + nseq + 1, dtype=torch.int32, device=row_start.device)
+        self.cs, self.sc, self.ids, self.zeros, self.ones = buf[:n + 1], buf[n + 1:n + 2 + nseq], buf[n + 2 + nseq:2 * n + 2 + nseq], \
+            buf[2 * n + 2 + nseq:3 * n + 2 + nseq], buf[3 * n + 2 + nseq:4 * n + 2 + nseq]
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_chunk_plan(row_start.data_ptr(), nseq, C, n, self.cs.data_ptr(), self.sc.data_ptr(), self.ids.data_ptr(),
+                                                            self.zeros.data_ptr(), self.ones.data_ptr(), _stream()), "hy_chunk_plan")
+
+
 def scan(mode: int, proj: torch.Tensor, qo: int, ko: int, vo: int, z: Optional[torch.Tensor], lower, fbias, tau: float, qscale: float,
-         heads: int, dim: int, vdim: int, row_start, slot, first_pos, state: torch.Tensor, act: torch.dtype) -> torch.Tensor:
-    """Gated linear recurrence over the rows of every sequence, continuing (and leaving) the fp32 state of its slot -> fp32 [T, heads * vdim]."""
+         heads: int, dim: int, vdim: int, row_start, slot, first_pos, state: torch.Tensor, act: torch.dtype, *, plans: Optional[dict] = None,
+         chunked: Optional[bool] = None) -> torch.Tensor:
+    """Gated linear recurrence over the rows of every sequence, continuing (and leaving) the fp32 state of its slot -> fp32 [T, heads * vdim].
+    The modes with a constant decay per head (SCAN_FIXED, SCAN_FIXED_SILU) run steps of SCAN_CHUNKED_FROM rows or more in chunks that are walked
+    side by side (every chunk from a zero state, a prefix over each sequence's chunks, then the chunk-start states' share of the outputs): the
+    same sums in another order.  plans: a dict that keeps the step's chunk plan between calls (the layers of one step share it); chunked
+    forces the choice."""
     _dev(proj, torch.float32, "scan.proj"); _dev(state, torch.float32, "scan.state")
     T = proj.shape[0]
     out = torch.empty(T, heads * vdim, dtype=torch.float32, device=proj.device)
     nseq = slot.numel()
-    if T and nseq:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_scan(mode, proj.data_ptr(), _rows(proj, "scan.proj"), qo, ko, vo, _p(z), 0 if z is None else _rows(z, "scan.z"),
-                                                      _p(lower), _p(fbias), float(tau), float(qscale), heads, dim, vdim, row_start.data_ptr(),
-                                                      slot.data_ptr(), first_pos.data_ptr(), nseq, state.data_ptr(), out.data_ptr(), act_code(act),
-                                                      _stream()), "hy_scan")
+    if not (T and nseq):
+        return out
+    lib, ld = _C.hybrid_lib(), _rows(proj, "scan.proj")
+
+    def run(m, rs, sl, fp, n, st):
+        _C.check_hybrid(lib.mi355_hy_scan(m, proj.data_ptr(), ld, qo, ko, vo, _p(z), 0 if z is None else _rows(z, "scan.z"), _p(lower), _p(fbias), float(tau),
+                                          float(qscale), heads, dim, vdim, rs.data_ptr(), sl.data_ptr(), fp.data_ptr(), n, st.data_ptr(), out.data_ptr(),
+                                          act_code(act), _stream()), "hy_scan")
+
+    fixed = mode in (SCAN_FIXED, SCAN_FIXED_SILU)
+    if chunked is None:
+        chunked = fixed and T >= SCAN_CHUNKED_FROM and T >= 2 * nseq
+    if not chunked:
+        run(mode, row_start, slot, first_pos, nseq, state)
+        return out
+    if not fixed or not state.is_contiguous() or state.shape[1:] != (heads, dim, vdim):
+        raise _C.Mi355Error(f"scan: the chunked form takes a constant decay per head and a contiguous state [slots, {heads}, {dim}, {vdim}]")
+    _dev(lower, torch.float32, "scan.decay")
+    C = SCAN_CHUNK
+    while (T // C + nseq + 1) * heads * dim * vdim * 4 > SCAN_CHUNK_BYTES and C < T:
+        C *= 2
+    key = (row_start.data_ptr(), T, nseq, C)
+    plan = plans.get(key) if plans is not None else None
+    if plan is None:
+        plan = ChunkPlan(row_start, T, nseq, C)
+        if plans is not None:
+            plans.clear()
+            plans[key] = plan
+    cstate = torch.empty(plan.max_chunks, heads, dim, vdim, dtype=torch.float32, device=proj.device)
+    run(mode, plan.cs, plan.ids, plan.zeros, plan.max_chunks, cstate)                       # 1: every chunk from a zero state
+    _C.check_hybrid(lib.mi355_hy_chunk_prefix(plan.cs.data_ptr(), plan.sc.data_ptr(), slot.data_ptr(), first_pos.data_ptr(), nseq, lower.data_ptr(), heads,
+                                              dim * vdim, cstate.data_ptr(), state.data_ptr(), _stream()), "hy_chunk_prefix")        # 2: states at the chunks' starts
+    run(mode + 4, plan.cs, plan.ids, plan.ones, plan.max_chunks, cstate)                    # 3: their share of the outputs
     return out
 
 

@@ -242,6 +242,54 @@ def test_lightning_scan_states_and_outputs(H, dim, vdim):
     assert float(sd[1].abs().max()) == 0.0 and float(sd[2].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("mode_silu,H,dim,vdim,chunk", [(True, 2, 16, 24, 64), (False, 1, 64, 64, 64), (True, 3, 20, 12, 128), (True, 2, 136, 72, 64), (False, 2, 8, 100, 64)])
+def test_chunked_form_of_the_fixed_decay_scan(mode_silu, H, dim, vdim, chunk):
+    """Long prompt portions walk their chunks side by side: against the token-by-token walk of the same kernel and against the definition, with
+    sequences that start fresh or continue a state, lengths on both sides of chunk borders, single rows between long ones, decays of 0 and 1."""
+    from rtp_llm_amd import hybrid_ops as hops
+    g = torch.Generator().manual_seed(dim * 7 + vdim)
+    lens, slots, first = [200, 1, 64, 65, 330, 2, 127], [6, 0, 3, 1, 5, 2, 4], [0, 9, 0, 40, 7, 0, 1]
+    T, hd, hv = sum(lens), H * dim, H * vdim
+    proj = torch.randn(T, 2 * hd + hv + 4, generator=g) * 0.7
+    qo, ko, vo = 0, hd, 2 * hd + 4
+    decay = torch.tensor([0.998, 0.5, 1.0][:H]) if H > 1 else torch.tensor([0.97])
+    if not mode_silu and H > 1:
+        decay[1] = 0.0
+    start = torch.randn(7, H, dim, vdim, generator=g)
+    act = O.silu if mode_silu else (lambda t: t)
+    rs = [0]
+    for n in lens:
+        rs.append(rs[-1] + n)
+    want, S_end = torch.zeros(T, hv, dtype=torch.float64), {}
+    for i, n in enumerate(lens):
+        S = [torch.zeros(dim, vdim, dtype=torch.float64) if first[i] == 0 else start[slots[i], j].double() for j in range(H)]
+        for t in range(rs[i], rs[i + 1]):
+            p = proj[t].double()
+            for j in range(H):
+                q, k = act(p[qo + j * dim:qo + (j + 1) * dim]), act(p[ko + j * dim:ko + (j + 1) * dim])
+                v = act(p[vo + j * vdim:vo + (j + 1) * vdim])
+                S[j] = float(decay[j]) * S[j] + torch.outer(k, v)
+                want[t, j * vdim:(j + 1) * vdim] = S[j].T @ q
+        S_end[i] = torch.stack(S)
+    I = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    mode = hops.SCAN_FIXED_SILU if mode_silu else hops.SCAN_FIXED
+    old = hops.SCAN_CHUNK
+    hops.SCAN_CHUNK = chunk
+    try:
+        for chunked in (True, False):
+            sd = start.clone().to(DEV)
+            plans = {}
+            out = hops.scan(mode, proj.to(DEV), qo, ko, vo, None, decay.to(DEV), None, 1.0, 1.0, H, dim, vdim, I(rs), I(slots), I(first), sd, torch.float32,
+                            plans=plans, chunked=chunked)
+            assert (len(plans) == 1) == chunked
+            scale = float(want.abs().max())
+            close(out, want, 2e-5 * scale)
+            for i in range(len(lens)):
+                close(sd[slots[i]], S_end[i], 2e-5 * float(S_end[i].abs().max()) + 1e-6)
+    finally:
+        hops.SCAN_CHUNK = old
+
+
 # ------------------------------------------------------------------------------------------------ mechanisms alone
 ALONE = {
     "plain": U.layer(),
