@@ -1243,12 +1243,12 @@ __global__ __launch_bounds__(256) void hy_delta_kernel(DeltaParams p) {
 }
 
 // per-head RMS norm over vdim with a plain weight (null: none; shared by the heads, or w_heads: one per head and channel, [H * vdim]), optional
-// gate (silu, or gate_sigmoid: sigmoid): one block per (row, head), a single wave for heads of up to 256 channels and four waves beyond (one
-// "head" that spans all heads of a row: a norm over the whole concatenation)
+// gate (silu, or gate_sigmoid: sigmoid): one block per (row, head), a single wave for heads of up to 256 channels and a wave per 256 channels
+// beyond, up to sixteen (one "head" that spans all heads of a row: a norm over the whole concatenation)
 template <typename T>
-__global__ __launch_bounds__(256) void hy_head_norm_kernel(const float* o, int H, int vdim, const T* w, float eps, const float* gate, int ldg, int goff, T* out,
+__global__ __launch_bounds__(1024) void hy_head_norm_kernel(const float* o, int H, int vdim, const T* w, float eps, const float* gate, int ldg, int goff, T* out,
                                                            int w_heads, int gate_sigmoid) {
-    __shared__ float red[4];
+    __shared__ float red[16];
     const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, NT = blockDim.x;
     const float* src = o + ((size_t)r * H + h) * vdim;
     float ss = 0.f;
@@ -1257,7 +1257,8 @@ __global__ __launch_bounds__(256) void hy_head_norm_kernel(const float* o, int H
     if (NT > 64) {
         if ((tid & 63) == 0) red[tid >> 6] = ss;
         __syncthreads();
-        ss = (red[0] + red[1]) + (red[2] + red[3]);
+        ss = 0.f;
+        for (int i = 0; i < (NT >> 6); ++i) ss += red[i];
     }
     const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
     for (int c = tid; c < vdim; c += NT) {
@@ -1855,7 +1856,7 @@ extern "C" int mi355_hy_head_norm(const float* o, int32_t rows, int32_t H, int32
 extern "C" int mi355_hy_head_norm_ex(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
                                      int32_t goff, void* out, int32_t w_heads, int32_t gate_sigmoid, int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(o && out && rows > 0 && H > 0 && vdim > 0, "hy_head_norm: bad argument");
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_head_norm_kernel<T>, dim3(rows, H), dim3(vdim > 256 ? 256 : 64), 0, (hipStream_t)stream, o, H, vdim, (const T*)w, eps,
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_head_norm_kernel<T>, dim3(rows, H), dim3(vdim > 256 ? std::min(1024, (vdim + 255) / 256 * 64) : 64), 0, (hipStream_t)stream, o, H, vdim, (const T*)w, eps,
                                               gate, ldg, goff, (T*)out, w_heads, gate_sigmoid));
     MI355_CHECK_LAUNCH("hy_head_norm_kernel");
     return MI355_OK;
