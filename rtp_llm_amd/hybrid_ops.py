@@ -356,8 +356,20 @@ def attn_tiles(q: torch.Tensor, scale: float, geom, chunk: int, sink: Optional[t
 
 
 SCAN_CHUNK = 64            # tokens per chunk of the chunked form of the fixed-decay recurrence ...
-SCAN_CHUNKED_FROM = 256    # ... which steps of at least this many rows (and two or more rows per sequence on average) take
+SCAN_CHUNKED_FROM = 256    # ... which a step takes when its longest sequence has at least this many rows and the walk would leave the chip idle
 SCAN_CHUNK_BYTES = 512 << 20
+SCAN_BLOCKS_AT_ONCE = 512  # blocks of the scan kernel the chip runs side by side (two per compute unit)
+
+
+def scan_prefers_chunks(T: int, nseq: int, max_rows: int, heads: int, vdim: int, C: int) -> bool:
+    """Whether the chunked form is expected to be faster: the token-by-token walk takes (rounds of blocks) x (rows of the longest sequence)
+    token steps, the chunked form two passes of (rounds of blocks over all chunks) x (chunk size)."""
+    longest = max_rows if max_rows > 0 else T - (nseq - 1)
+    if longest < SCAN_CHUNKED_FROM:
+        return False
+    per = heads * ((vdim + 63) // 64)
+    rounds = lambda blocks: -(-blocks // SCAN_BLOCKS_AT_ONCE)
+    return 2 * rounds((T // C + nseq + 1) * per) * C < rounds(nseq * per) * longest
 
 
 class ChunkPlan:
@@ -375,12 +387,13 @@ class ChunkPlan:
 
 def scan(mode: int, proj: torch.Tensor, qo: int, ko: int, vo: int, z: Optional[torch.Tensor], lower, fbias, tau: float, qscale: float,
          heads: int, dim: int, vdim: int, row_start, slot, first_pos, state: torch.Tensor, act: torch.dtype, *, plans: Optional[dict] = None,
-         chunked: Optional[bool] = None) -> torch.Tensor:
+         chunked: Optional[bool] = None, max_rows: int = 0) -> torch.Tensor:
     """Gated linear recurrence over the rows of every sequence, continuing (and leaving) the fp32 state of its slot -> fp32 [T, heads * vdim].
-    The modes with a constant decay per head (SCAN_FIXED, SCAN_FIXED_SILU) run steps of SCAN_CHUNKED_FROM rows or more in chunks that are walked
-    side by side (every chunk from a zero state, a prefix over each sequence's chunks, then the chunk-start states' share of the outputs): the
-    same sums in another order.  plans: a dict that keeps the step's chunk plan between calls (the layers of one step share it); chunked
-    forces the choice."""
+    The modes with a constant decay per head (SCAN_FIXED, SCAN_FIXED_SILU) run long prompt portions in chunks that are walked side by side
+    (every chunk from a zero state, a prefix over each sequence's chunks, then the chunk-start states' share of the outputs): the same sums in
+    another order.  They do so when that is expected to be faster (scan_prefers_chunks: few long sequences; max_rows = the rows of the step's
+    longest sequence when the caller knows it).  plans: a dict that keeps the step's chunk plan between calls (the layers of one step share
+    it); chunked forces the choice."""
     _dev(proj, torch.float32, "scan.proj"); _dev(state, torch.float32, "scan.state")
     T = proj.shape[0]
     out = torch.empty(T, heads * vdim, dtype=torch.float32, device=proj.device)
@@ -396,7 +409,7 @@ def scan(mode: int, proj: torch.Tensor, qo: int, ko: int, vo: int, z: Optional[t
 
     fixed = mode in (SCAN_FIXED, SCAN_FIXED_SILU)
     if chunked is None:
-        chunked = fixed and T >= SCAN_CHUNKED_FROM and T >= 2 * nseq
+        chunked = fixed and scan_prefers_chunks(T, nseq, max_rows, heads, vdim, SCAN_CHUNK)
     if not chunked:
         run(mode, row_start, slot, first_pos, nseq, state)
         return out

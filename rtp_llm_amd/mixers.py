@@ -142,6 +142,7 @@ class StepBatch:
     prev: Optional[torch.Tensor] = None        # the token before each row in its sequence (-1 for a sequence's first token): bigram embeddings
     host: Optional[torch.Tensor] = None        # the pinned buffer all index fields were uploaded from (one copy per step)
     plans: dict = field(default_factory=dict)  # what the step's layers share beyond the index arrays (the chunk plan of the fixed-decay recurrences)
+    max_rows: int = 0                          # rows of the step's longest sequence when the host knows them (0: unknown)
 
 
 def rotary_table(rot: RotarySpec, device):
@@ -437,7 +438,7 @@ class Retention:
         hops.rotary(proj, [(self.qo, s.heads, s.dim, 1.0), (self.ko, s.heads, s.dim, 1.0 / math.sqrt(s.dim))], rot.dims if rot else 0,
                     hops.LAYOUTS[rot.layout] if rot else 0, self.freq, self.mag, batch.pos)
         o = hops.scan(hops.SCAN_FIXED, proj, self.qo, self.ko, self.vo, None, self.decay, None, 1.0, 1.0, s.heads, s.dim, s.vdim,
-                      batch.row_start, batch.slot, batch.first_pos, state, self.act, plans=batch.plans)
+                      batch.row_start, batch.slot, batch.first_pos, state, self.act, plans=batch.plans, max_rows=batch.max_rows)
         o = hops.head_norm(o, s.heads, s.vdim, None, self.eps, proj, self.go, out_dtype=self.act)
         return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
 
@@ -487,7 +488,7 @@ class LightningAttention:
         if proj is None:
             proj = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
         o = hops.scan(hops.SCAN_FIXED_SILU, proj, self.qo, self.ko, self.vo, None, self.decay, None, 1.0, 1.0, s.heads, s.dim, s.vdim,
-                      batch.row_start, batch.slot, batch.first_pos, state, self.act, plans=batch.plans)
+                      batch.row_start, batch.slot, batch.first_pos, state, self.act, plans=batch.plans, max_rows=batch.max_rows)
         o = hops.head_norm(o, 1, s.heads * s.vdim, self.norm, self.eps, proj, self.go, gate_act="sigmoid")
         return hops.dense_linear(o, self.w_o, out_dtype=torch.float32) if out_proj else o
 

@@ -103,6 +103,7 @@ class ServingEngine:
                 host[o:o + len(part)] = torch.tensor(part, dtype=torch.int32)
         batch = self.batch_views(host.to(self.device, non_blocking=True), [len(part) for part in parts], len(tables), width)
         batch.host = host
+        batch.max_rows = max(b - a for a, b in zip(row_start[:-1], row_start[1:]))
         return batch
 
     @staticmethod
@@ -139,6 +140,7 @@ class ServingEngine:
             buf.copy_(batch.host)
             nseq, width = key
             static = self.batch_views(buf, [nseq, nseq, nseq, nseq + 1, nseq, nseq, nseq * width, nseq, nseq, nseq, nseq], nseq, width)
+            static.max_rows = 1
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
