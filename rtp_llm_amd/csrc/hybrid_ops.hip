@@ -1456,15 +1456,16 @@ __device__ __forceinline__ void hy_route_token(bool active, const float* zr, flo
         if (active) for (int g = lane; g < groups; g += 64) gb[g] = INFINITY;
         __syncthreads();
     }
+    // sigmoid scores are ranked by their logits (the same order, and it survives where the fp32 sigmoid rounds to one)
     for (int k = 0; k < top; ++k) {
-        float bv = -2.f; int bi = 0x7fffffff;
+        float bv = -INFINITY; int bi = 0x7fffffff;
         if (active)
             for (int e = lane; e < E; e += 64) {
-                const float v = sc[e];
-                if (v >= 0.f && gb[e / per] == INFINITY && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }
+                const float v = rm.sigmoid ? zr[e] : sc[e];
+                if (sc[e] >= 0.f && gb[e / per] == INFINITY && (bi == 0x7fffffff || v > bv || (v == bv && e < bi))) { bv = v; bi = e; }
             }
         hy_wave_argmax(bv, bi);
-        if (active && lane == 0) { ids[k] = bi; wts[k] = bv * rm.wscale; sc[bi] = -1.f; }     // taken
+        if (active && lane == 0) { ids[k] = bi; wts[k] = sc[bi] * rm.wscale; sc[bi] = -1.f; }     // taken
         __syncthreads();
     }
 }

@@ -168,6 +168,17 @@ def test_sigmoid_router_with_groups_ranked_by_their_two_best(E, count, keep, top
         assert differs > 0, "no token tells a ranking by two best from a ranking by the best"
 
 
+def test_sigmoid_router_ranks_by_logit_where_the_sigmoid_rounds_to_one():
+    """Logits beyond 17 all have an fp32 sigmoid of exactly one; the order of the logits still decides (one group, so no group sums tie)."""
+    from rtp_llm_amd import hybrid_ops as hops
+    g = torch.Generator().manual_seed(77)
+    z = torch.randn(40, 12, generator=g) * 3 + 30.0
+    assert float(torch.sigmoid(z).min()) == 1.0
+    ids, wts = hops.moe_route(z.to(DEV), 1, 1, 5, sigmoid=True, group_top=2, scale=2.0)
+    assert ids.cpu().tolist() == z.topk(5, dim=1).indices.tolist()
+    assert float((wts - 2.0).abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("H,G,dim", [(4, 1, 16), (3, 3, 20), (2, 1, 64), (5, 5, 8), (8, 2, 128)])
 def test_query_and_key_norm_over_all_heads_at_once(H, G, dim):
     """attn_prep with the norm over the whole projection: the queries come back normed and turned, the keys land in their pages."""
