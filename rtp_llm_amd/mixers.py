@@ -419,11 +419,15 @@ class Retention:
             raise ValueError(f"retention: {len(s.decay)} decays for {s.heads} heads")
         hd = s.heads * s.dim
         self.w_in = torch.cat([weights["q"], weights["k"], weights["v"], weights["g"]], 0).contiguous()
+        self.b_in = None
         self.qo, self.ko, self.vo, self.go = 0, hd, 2 * hd, 2 * hd + s.heads * s.vdim
         self.decay = torch.tensor([float(a) for a in s.decay], dtype=torch.float32, device=device)
         self.w_o = weights["o"].contiguous()
         self.act = self.w_o.dtype
         self.freq, self.mag = rotary_table(s.rot, device) if s.rot is not None else (None, 1.0)
+
+    def cache_kind(self):
+        return "state"
 
     def state_shape(self):
         s = self.spec
